@@ -128,6 +128,64 @@ class BiasedAttentionSpec(MixerSpec):
 
 
 @dataclass(frozen=True)
+class LatentAttentionSpec(MixerSpec):
+    """Causal softmax attention whose keys and values are made from one small latent row per position.
+
+    ``cq = rms(q_down x) * q_norm``, ``q = q_up cq`` (per head ``head_dim`` plain elements, then ``rot_dim`` that
+    are rotated); ``kv_down x = [c' | r]`` with ``c = rms(c') * kv_norm`` (``kv_rank`` elements) and ``r``
+    (``rot_dim`` elements, rotated, shared by the heads).  Head h's key is ``[k_up_h c | r]``, its value
+    ``v_up_h c``; the score is ``scale * q . k``.  The cache holds ``[c | r]`` per position and nothing per head.
+    The heads side by side are multiplied by ``sigmoid(gate_proj x)`` where a gate is named.  Without ``kv_down``
+    the mixer reads the latent rows of the memory its run-order entry names, with its own ``k_up`` and ``v_up``.
+    ``position`` rotates the first ``rotary_dim`` of the ``rot_dim`` elements (pairs i, i + rotary_dim / 2)."""
+    hidden: int = 0
+    n_heads: int = 0
+    head_dim: int = 0              # elements of a query/key head that are not rotated
+    rot_dim: int = 0               # elements that are (queries: per head; keys: one part for all heads)
+    v_head_dim: int = 0
+    q_rank: int = 0
+    kv_rank: int = 0
+    scale: float = 1.0
+    norm_eps: float = 1e-5         # of the latents' norms
+    position: PositionSpec = PositionSpec("none")
+    q_down: str = ""               # [q_rank, hidden]
+    q_norm: str = ""               # [q_rank]
+    q_up: str = ""                 # [heads * (head_dim + rot_dim), q_rank]
+    kv_down: str = ""              # [kv_rank + rot_dim, hidden]; "": another memory's latent rows are read
+    kv_norm: str = ""              # [kv_rank]
+    k_up: str = ""                 # [heads * head_dim, kv_rank]
+    v_up: str = ""                 # [heads * v_head_dim, kv_rank]
+    gate_proj: str = ""            # [heads * v_head_dim, hidden]; "": no gate
+    o_proj: str = ""               # [hidden, heads * v_head_dim]
+
+
+@dataclass(frozen=True)
+class Mamba2Spec(MixerSpec):
+    """A state-space mixer with one decay per head and token (state [heads, state, v_head_dim]).
+
+    ``in_proj x = [z | xs | B | C | dt]`` (``heads * v_head_dim`` twice, ``groups * state`` twice, ``heads``);
+    ``xs, B, C`` pass one short causal convolution with a bias and SiLU; ``dt = softplus(dt + dt_bias)``;
+    head h (group ``h // (heads / groups)``): ``S <- exp(-exp(a_log_h) dt) S + dt B xs^T``, ``y = S^T C + d_skip_h xs``;
+    ``y * silu(z)`` is divided by its root mean square in ``norm_groups`` equal parts, times ``out_norm``."""
+    hidden: int = 0
+    n_heads: int = 0
+    v_head_dim: int = 0
+    state: int = 0
+    groups: int = 1
+    conv_taps: int = 1
+    norm_groups: int = 1
+    norm_eps: float = 1e-5
+    in_proj: str = ""
+    conv: str = ""                 # [heads * v_head_dim + 2 * groups * state, taps], the last column is the current token's
+    conv_bias: str = ""            # "": none
+    dt_bias: str = ""              # [heads]
+    a_log: str = ""                # [heads]
+    d_skip: str = ""               # [heads]
+    out_norm: str = ""             # [heads * v_head_dim]
+    o_proj: str = ""
+
+
+@dataclass(frozen=True)
 class GatedDeltaSpec(MixerSpec):
     """Delta rule with a decay per head and key channel (state [heads, head_dim, v_head_dim])."""
     hidden: int = 0
@@ -209,6 +267,9 @@ class GatedFfnSpec(FeedForwardSpec):
     gate_bias: str = ""            # names of the products' bias vectors; "": none
     up_bias: str = ""
     down_bias: str = ""
+    # ``swish_clamped``: g = min(gate, act_limit), u = clamp(up, -act_limit, act_limit), g sigmoid(act_alpha g) (u + 1)
+    act_limit: float = 0.0
+    act_alpha: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -218,7 +279,13 @@ class RoutedFfnSpec(FeedForwardSpec):
     the softmax over all outputs; the ``top`` outputs with the largest score + correction are chosen, among
     the ``keep_groups`` best of ``groups`` equal groups of neighbouring outputs (a group counts by its largest
     score + correction); a chosen expert's weight is its score times ``route_scale``.  ``shared``: an expert
-    that every token runs through, added."""
+    that every token runs through, added; with ``shared_gate`` [1, hidden] it is first multiplied by
+    ``sigmoid(shared_gate . x)``, one number per token.
+
+    ``score="softmax_top"`` instead: the router's logits plus ``correction`` (a bias of the logits here) decide, the
+    ``top`` largest are chosen, and the weights are the softmax over the chosen logits alone, times ``route_scale``
+    (no groups).  ``act_limit`` and ``act_alpha`` are the activation's numbers where it has some
+    (``swish_clamped``, see :class:`GatedFfnSpec`)."""
     hidden: int = 0
     intermediate: int = 0          # of every expert
     n_experts: int = 0
@@ -235,6 +302,10 @@ class RoutedFfnSpec(FeedForwardSpec):
     up_name: str = "up"
     down_name: str = "down"
     shared: Optional[GatedFfnSpec] = None
+    score: str = "softmax_all"     # | "softmax_top"
+    shared_gate: str = ""          # [1, hidden]; "": the shared expert is added as it is
+    act_limit: float = 0.0
+    act_alpha: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -244,6 +315,7 @@ class LayerSpec:
     ``"sandwich"``: h += post_mixer_norm(mixer(pre_mixer_norm(h)));
                     h += post_ffn_norm(ffn(pre_ffn_norm(h)))
     ``"prenorm"``:  the same without the two post norms.
+    ``"postnorm"``: h += post_mixer_norm(mixer(h));  h += post_ffn_norm(ffn(h)): the sublayers read the stream itself.
     """
     kind: str
     mixer: MixerSpec
@@ -287,6 +359,7 @@ class ModelSpec:
     # soft-capped to +-``logit_softcap`` (cap * tanh(x / cap)) if that is above zero
     logit_scale: float = 1.0
     logit_softcap: float = 0.0
+    embed_norm: Optional[NormSpec] = None    # a norm on the embedding rows before the first layer
     extra: Dict[str, object] = field(default_factory=dict)
 
     def default_order(self) -> List[RunEntry]:

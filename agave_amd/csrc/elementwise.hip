@@ -699,6 +699,7 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 // 1 silu, x / (1 + exp(-x)); 2 gelu with the error function; 3 relu.  Another one is another case
 // here; only the tanh form also ends the matrix-core products (gemm_mfma.hip).
 #define AGAVE_GATE_ACTS 4
+#define AGAVE_GATE_SWISH_CLAMPED 6     // a gated form with two numbers of its own, known to gated_act only
 __device__ __forceinline__ float gate_act(float x, int act) {
     switch (act) {
         case 0: return gelu_tanh(x);
@@ -710,29 +711,35 @@ __device__ __forceinline__ float gate_act(float x, int act) {
 
 template <typename T>
 __global__ void gated_act_kernel(const T* __restrict__ gate, long ldg, const T* __restrict__ up, long ldu,
-                                 T* __restrict__ out, long ldo, long total, int ff, int act) {
+                                 T* __restrict__ out, long ldo, long total, int ff, int act, float p0, float p1) {
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
         const long r = idx / ff;
         const int c = (int)(idx % ff);
         const float g = ld(gate + r * ldg + c), u = ld(up + r * ldu + c);
-        st(out + r * ldo + c, gate_act(g, act) * u);
+        if (act == AGAVE_GATE_SWISH_CLAMPED) {
+            // g' = min(g, p0), u' = clamp(u, -p0, p0);  g' sigmoid(p1 g') (u' + 1)
+            const float gc = fminf(g, p0), uc = fminf(fmaxf(u, -p0), p0);
+            st(out + r * ldo + c, gc / (1.0f + expf(-p1 * gc)) * (uc + 1.0f));
+        } else {
+            st(out + r * ldo + c, gate_act(g, act) * u);
+        }
     }
 }
 
 // out = act(gate) * up, row by row
-extern "C" int agave_gated_act(int dtype, int act, const void* gate, long ldg, const void* up, long ldu, void* out,
-                               long ldo, int n_rows, int ff, hipStream_t stream) {
+extern "C" int agave_gated_act(int dtype, int act, float p0, float p1, const void* gate, long ldg, const void* up, long ldu,
+                               void* out, long ldo, int n_rows, int ff, hipStream_t stream) {
     AGAVE_CHECK(n_rows >= 0 && ff > 0, "gated_act: bad sizes rows=%d ff=%d", n_rows, ff);
-    AGAVE_CHECK(act >= 0 && act < AGAVE_GATE_ACTS, "gated_act: unknown activation %d", act);
+    AGAVE_CHECK((act >= 0 && act < AGAVE_GATE_ACTS) || act == AGAVE_GATE_SWISH_CLAMPED, "gated_act: unknown activation %d", act);
     AGAVE_CHECK(ldg >= ff && ldu >= ff && ldo >= ff, "gated_act: a row stride is below %d", ff);
     if (n_rows == 0) return 0;
     const long total = (long)n_rows * ff;
     long blocks = (total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     if (dtype == AGAVE_F32)
-        gated_act_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)gate, ldg, (const float*)up, ldu, (float*)out, ldo, total, ff, act);
+        gated_act_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)gate, ldg, (const float*)up, ldu, (float*)out, ldo, total, ff, act, p0, p1);
     else if (dtype == AGAVE_BF16)
-        gated_act_kernel<bf16><<<(int)blocks, 256, 0, stream>>>((const bf16*)gate, ldg, (const bf16*)up, ldu, (bf16*)out, ldo, total, ff, act);
+        gated_act_kernel<bf16><<<(int)blocks, 256, 0, stream>>>((const bf16*)gate, ldg, (const bf16*)up, ldu, (bf16*)out, ldo, total, ff, act, p0, p1);
     else
         AGAVE_CHECK(false, "gated_act: unknown dtype %d", dtype);
     AGAVE_LAUNCH_CHECK("gated_act");
@@ -811,7 +818,7 @@ extern "C" int agave_unary_act(int dtype, int act, float p0, float p1, const voi
 
 extern "C" int agave_geglu(int dtype, const void* gate, long ldg, const void* up, long ldu, void* out, long ldo,
                            int n_rows, int ff, hipStream_t stream) {
-    return agave_gated_act(dtype, 0, gate, ldg, up, ldu, out, ldo, n_rows, ff, stream);
+    return agave_gated_act(dtype, 0, 0.f, 0.f, gate, ldg, up, ldu, out, ldo, n_rows, ff, stream);
 }
 
 // ------------------------------------------------------------------ a product's bias

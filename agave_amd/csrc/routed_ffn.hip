@@ -7,6 +7,10 @@
 //   chosen (the lower index wins a tie); the weight of a chosen output is s * scale.
 //   Outputs e >= E are identity experts: their result is the feed-forward's input row itself.
 //   Expert e < E: W_down[e] (act(W_gate[e] x) * (W_up[e] x)).
+//   The other way of scoring (mode 1): the logits z + bias decide, the `top` largest are chosen, and the weights are
+//   the softmax over the chosen logits alone, times scale.
+//   The router matrix may carry further rows behind its R outputs (`extra`): their products with the token are handed
+//   out as they are (the logit of a gate on the shared expert), so that they cost no kernel of their own.
 //
 // A (token, slot) pair p = t * top + slot names one chosen output.  The plain kernels take the pairs
 // as they come (a wave per pair and output column).  The matrix-core kernels take them sorted by
@@ -118,14 +122,16 @@ template <typename T, bool WIDE, int RR>
 __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ router,
                                                           const float* __restrict__ correction, int N, int K, int R, int groups,
                                                           int keep, int top, float scale, int* __restrict__ choice,
-                                                          float* __restrict__ weight) {
-    extern __shared__ float zs[];                      // [RR][R], then the corrections [R]
+                                                          float* __restrict__ weight, int mode, int extra,
+                                                          float* __restrict__ extra_out) {
+    extern __shared__ float zs[];                      // [RR][R + extra], then the corrections [R]
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    float* corr = zs + RR * R;                 // (read many times by the one thread that chooses: from LDS, not memory)
+    const int Rt = R + extra;
+    float* corr = zs + RR * Rt;                // (read many times by the one thread that chooses: from LDS, not memory)
     for (int e = threadIdx.x; e < R; e += blockDim.x) corr[e] = correction ? correction[e] : 0.f;
     const int t0 = blockIdx.x * RR;
     const int rows = min(RR, N - t0);
-    for (int r = w; r < R; r += nw) {
+    for (int r = w; r < Rt; r += nw) {
         const float* wr = router + (size_t)r * K;
         float acc[RR];
 #pragma unroll
@@ -157,15 +163,53 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
 #pragma unroll
         for (int i = 0; i < RR; ++i) {
             const float sum = wave_sum(acc[i]);
-            if (lane == 0) zs[i * R + r] = sum;
+            if (lane == 0) zs[i * Rt + r] = sum;
         }
     }
     __syncthreads();
+    for (int i = threadIdx.x; i < rows * extra; i += blockDim.x)
+        extra_out[(size_t)(t0 + i / extra) * extra + i % extra] = zs[(i / extra) * Rt + R + i % extra];
     // the choice: a wave per token, the lanes along the outputs
     const int gs = R / groups;
     for (int i = w; i < rows; i += nw) {
-        float* sr = zs + (size_t)i * R;
+        float* sr = zs + (size_t)i * Rt;
         const int t = t0 + i;
+        if (mode == 1) {
+            // the largest logits (bias added) are chosen, the lower index among equals; a chosen place is marked by
+            // -infinity; lane r keeps round r's logit, and the weights are the softmax over those (top <= 64)
+            for (int e = lane; e < R; e += 64) sr[e] += corr[e];
+            __builtin_amdgcn_wave_barrier();
+            int my_choice = 0;
+            float my_logit = 0.f, first_v = 0.f, sum = 0.f;
+            for (int r = 0; r < top; ++r) {
+                float best_v = -INFINITY;
+                int best = -1;
+                for (int e = lane; e < R; e += 64) {
+                    const float se = sr[e];
+                    if (se == -INFINITY) continue;
+                    if (best < 0 || se > best_v) {
+                        best = e;
+                        best_v = se;
+                    }
+                }
+                const float top_v = wave_max(best >= 0 ? best_v : -INFINITY);
+                int chosen = (int)(-wave_max((best >= 0 && best_v == top_v) ? -(float)best : -INFINITY));
+                if (chosen < 0 || chosen >= R) chosen = 0;          // (every open logit is -infinity or not a number)
+                if (r == 0) first_v = top_v;
+                sum += expf(top_v - first_v);
+                if (r == lane) {
+                    my_choice = chosen;
+                    my_logit = top_v;
+                }
+                if (lane == 0) sr[chosen] = -INFINITY;
+                __builtin_amdgcn_wave_barrier();
+            }
+            if (lane < top) {
+                choice[(size_t)t * top + lane] = my_choice;
+                weight[(size_t)t * top + lane] = expf(my_logit - first_v) / sum * scale;
+            }
+            continue;
+        }
         float mx = -INFINITY;
         for (int e = lane; e < R; e += 64) mx = fmaxf(mx, sr[e]);
         mx = wave_max(mx);
@@ -230,8 +274,10 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
 }
 
 extern "C" int agave_route_rows(int dtype, const void* x, long ldx, const float* router, const float* correction, int N, int K,
-                                int R, int groups, int keep, int top, float scale, int* choice, float* weight,
-                                hipStream_t stream) {
+                                int R, int groups, int keep, int top, float scale, int* choice, float* weight, int mode,
+                                int extra, float* extra_out, hipStream_t stream) {
+    AGAVE_CHECK(mode == 0 || (mode == 1 && top <= 64 && groups == 1), "route_rows: the softmax over the chosen logits takes at most 64 of them and no groups");
+    AGAVE_CHECK(extra >= 0 && extra <= 64 && (extra == 0 || extra_out), "route_rows: %d further rows of the router (0 to 64, with a place for their products)", extra);
     AGAVE_CHECK(N >= 0 && K > 0 && R > 0 && R <= ROUTE_MAX, "route_rows: %d router outputs (1 to %d)", R, ROUTE_MAX);
     AGAVE_CHECK(groups > 0 && groups <= 64 && R % groups == 0, "route_rows: %d outputs in %d groups (equal groups, at most 64)", R, groups);
     AGAVE_CHECK(keep > 0 && keep <= groups, "route_rows: %d of %d groups kept", keep, groups);
@@ -242,15 +288,15 @@ extern "C" int agave_route_rows(int dtype, const void* x, long ldx, const float*
     AGAVE_CHECK(dtype == AGAVE_F32 || dtype == AGAVE_BF16, "route_rows: unknown dtype %d", dtype);
     const bool f32 = dtype == AGAVE_F32;
     if (N <= 64) {
-        const size_t lds = (size_t)2 * R * sizeof(float);
-#define ROUTE_GO(T_, W_) route_rows_kernel<T_, W_, 1><<<N, 1024, lds, stream>>>((const T_*)x, ldx, router, correction, N, K, R, groups, keep, top, scale, choice, weight)
+        const size_t lds = (size_t)(2 * R + extra) * sizeof(float);
+#define ROUTE_GO(T_, W_) route_rows_kernel<T_, W_, 1><<<N, 1024, lds, stream>>>((const T_*)x, ldx, router, correction, N, K, R, groups, keep, top, scale, choice, weight, mode, extra, extra_out)
         if (f32 && wide) ROUTE_GO(float, true); else if (f32) ROUTE_GO(float, false); else if (wide) ROUTE_GO(bf16, true); else ROUTE_GO(bf16, false);
 #undef ROUTE_GO
     } else {
         const int blocks = (N + 7) / 8;
-        const size_t lds = (size_t)9 * R * sizeof(float);
+        const size_t lds = (size_t)(9 * R + 8 * extra) * sizeof(float);
         const int threads = blocks <= 512 ? 1024 : 256;        // (more waves to share the outputs while they all fit the chip at once)
-#define ROUTE_GO(T_, W_) route_rows_kernel<T_, W_, 8><<<blocks, threads, lds, stream>>>((const T_*)x, ldx, router, correction, N, K, R, groups, keep, top, scale, choice, weight)
+#define ROUTE_GO(T_, W_) route_rows_kernel<T_, W_, 8><<<blocks, threads, lds, stream>>>((const T_*)x, ldx, router, correction, N, K, R, groups, keep, top, scale, choice, weight, mode, extra, extra_out)
         if (f32 && wide) ROUTE_GO(float, true); else if (f32) ROUTE_GO(float, false); else if (wide) ROUTE_GO(bf16, true); else ROUTE_GO(bf16, false);
 #undef ROUTE_GO
     }
@@ -259,6 +305,16 @@ extern "C" int agave_route_rows(int dtype, const void* x, long ldx, const float*
 }
 
 // ------------------------------------------------------------------ activations of the experts' gates
+// act(gate) * up for activations 0 to 3; 6 ("swish_clamped"): g = min(gate, p0), u = clamp(up, -p0, p0),
+// g sigmoid(p1 g) (u + 1)
+__device__ __forceinline__ float expert_act(float x, int act);
+__device__ __forceinline__ float expert_gated(float gate, float up, int act, float p0, float p1) {
+    if (act == 6) {
+        const float g = fminf(gate, p0), u = fminf(fmaxf(up, -p0), p0);
+        return g / (1.0f + expf(-p1 * g)) * (u + 1.0f);
+    }
+    return expert_act(gate, act) * up;
+}
 __device__ __forceinline__ float expert_act(float x, int act) {
     switch (act) {
         case 0: { const float c = 0.7978845608028654f; return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x * x * x))); }
@@ -273,7 +329,8 @@ __device__ __forceinline__ float expert_act(float x, int act) {
 template <typename T>
 __global__ __launch_bounds__(256) void routed_gate_up_plain_kernel(const T* __restrict__ x, long ldx, const int* __restrict__ choice,
                                                                    const T* __restrict__ wg, const T* __restrict__ wu,
-                                                                   T* __restrict__ act_out, int top, int E, int ff, int K, int act) {
+                                                                   T* __restrict__ act_out, int top, int E, int ff, int K, int act,
+                                                                   float p0, float p1) {
     const int p = blockIdx.x;
     const int e = choice[p];
     if (e < 0 || e >= E) return;
@@ -297,7 +354,7 @@ __global__ __launch_bounds__(256) void routed_gate_up_plain_kernel(const T* __re
         T tg, tu;
         st(&tg, ag);
         st(&tu, au);
-        st(act_out + (size_t)p * ff + f, expert_act(ld(&tg), act) * ld(&tu));
+        st(act_out + (size_t)p * ff + f, expert_gated(ld(&tg), ld(&tu), act, p0, p1));
     }
 }
 
@@ -325,8 +382,8 @@ __global__ __launch_bounds__(256) void routed_down_plain_kernel(const T* __restr
 template <typename T>
 __global__ void routed_combine_kernel(const float* __restrict__ y, const int* __restrict__ place, const int* __restrict__ choice,
                                       const float* __restrict__ weight, const T* __restrict__ x, long ldx,
-                                      const T* __restrict__ shared, long lds, T* __restrict__ out, long ldo, int N, int top,
-                                      int E, int hidden) {
+                                      const T* __restrict__ shared, long lds, const float* __restrict__ shared_gate,
+                                      T* __restrict__ out, long ldo, int N, int top, int E, int hidden) {
     const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (long)N * hidden) return;
     const int t = (int)(idx / hidden), c = (int)(idx % hidden);
@@ -346,26 +403,27 @@ __global__ void routed_combine_kernel(const float* __restrict__ y, const int* __
         const float yv = y ? y[(size_t)row * hidden + c] : 0.f;
         acc = fmaf(w, e >= E ? xv : (expert ? yv : 0.f), acc);
     }
-    if (shared) acc += sv;
+    // (the shared expert's row, times the sigmoid of a logit per token where it has a gate)
+    if (shared) acc = shared_gate ? fmaf(1.0f / (1.0f + expf(-shared_gate[t])), sv, acc) : acc + sv;
     st(out + (size_t)t * ldo + c, acc);
 }
 
 extern "C" int agave_routed_experts_plain(int dtype, const void* x, long ldx, const int* choice, const void* wg, const void* wu,
                                           const void* wd, void* act_rows, float* y, int N, int top, int E, int ff, int hidden,
-                                          int act, hipStream_t stream) {
+                                          int act, float p0, float p1, hipStream_t stream) {
     AGAVE_CHECK(N >= 0 && top > 0 && E >= 0 && ff > 0 && hidden > 0, "routed_experts: bad sizes");
-    AGAVE_CHECK(act >= 0 && act < 4, "routed_experts: unknown activation %d", act);
+    AGAVE_CHECK((act >= 0 && act < 4) || act == 6, "routed_experts: unknown activation %d", act);
     AGAVE_CHECK(x && choice && act_rows && y && ldx >= hidden && (E == 0 || (wg && wu && wd)), "routed_experts: bad buffers");
     AGAVE_CHECK((ff + 3) / 4 <= 65535 && (hidden + 3) / 4 <= 65535, "routed_experts: too many columns for the grid");
     if (N == 0 || E == 0) return 0;
     const dim3 g1(N * top, (ff + 3) / 4), g2(N * top, (hidden + 3) / 4);
     if (dtype == AGAVE_F32) {
         routed_gate_up_plain_kernel<float><<<g1, 256, 0, stream>>>((const float*)x, ldx, choice, (const float*)wg, (const float*)wu,
-                                                                   (float*)act_rows, top, E, ff, hidden, act);
+                                                                   (float*)act_rows, top, E, ff, hidden, act, p0, p1);
         routed_down_plain_kernel<float><<<g2, 256, 0, stream>>>((const float*)act_rows, choice, (const float*)wd, y, E, ff, hidden);
     } else if (dtype == AGAVE_BF16) {
         routed_gate_up_plain_kernel<bf16><<<g1, 256, 0, stream>>>((const bf16*)x, ldx, choice, (const bf16*)wg, (const bf16*)wu,
-                                                                  (bf16*)act_rows, top, E, ff, hidden, act);
+                                                                  (bf16*)act_rows, top, E, ff, hidden, act, p0, p1);
         routed_down_plain_kernel<bf16><<<g2, 256, 0, stream>>>((const bf16*)act_rows, choice, (const bf16*)wd, y, E, ff, hidden);
     } else
         AGAVE_CHECK(false, "routed_experts: unknown dtype %d", dtype);
@@ -374,8 +432,8 @@ extern "C" int agave_routed_experts_plain(int dtype, const void* x, long ldx, co
 }
 
 extern "C" int agave_routed_combine(int dtype, const float* y, const int* place, const int* choice, const float* weight,
-                                    const void* x, long ldx, const void* shared, long lds, void* out, long ldo, int N, int top,
-                                    int E, int hidden, hipStream_t stream) {
+                                    const void* x, long ldx, const void* shared, long lds, const float* shared_gate, void* out,
+                                    long ldo, int N, int top, int E, int hidden, hipStream_t stream) {
     AGAVE_CHECK(N >= 0 && top > 0 && hidden > 0, "routed_combine: bad sizes");
     AGAVE_CHECK(choice && weight && x && out && (E == 0 || y) && ldx >= hidden && ldo >= hidden && (!shared || lds >= hidden),
                 "routed_combine: bad buffers");
@@ -384,10 +442,10 @@ extern "C" int agave_routed_combine(int dtype, const float* y, const int* place,
     const int blocks = (int)((total + 255) / 256);
     if (dtype == AGAVE_F32)
         routed_combine_kernel<float><<<blocks, 256, 0, stream>>>(y, place, choice, weight, (const float*)x, ldx, (const float*)shared,
-                                                                 lds, (float*)out, ldo, N, top, E, hidden);
+                                                                 lds, shared_gate, (float*)out, ldo, N, top, E, hidden);
     else if (dtype == AGAVE_BF16)
         routed_combine_kernel<bf16><<<blocks, 256, 0, stream>>>(y, place, choice, weight, (const bf16*)x, ldx, (const bf16*)shared,
-                                                                lds, (bf16*)out, ldo, N, top, E, hidden);
+                                                                lds, shared_gate, (bf16*)out, ldo, N, top, E, hidden);
     else
         AGAVE_CHECK(false, "routed_combine: unknown dtype %d", dtype);
     AGAVE_LAUNCH_CHECK("routed_combine");
@@ -461,7 +519,7 @@ template <int MI, int NJ, bool GATED>
 __global__ __launch_bounds__(256) void routed_product_mfma_kernel(const bf16* __restrict__ x, long ldx, const int* __restrict__ sorted_pair,
                                                                   const int* __restrict__ tile_expert, const bf16* __restrict__ w0,
                                                                   const bf16* __restrict__ w1, void* __restrict__ out_, int top,
-                                                                  int n_out, int K, int act, int wpacked) {
+                                                                  int n_out, int K, int act, int wpacked, float p0, float p1) {
     const int e = tile_expert[blockIdx.x];
     if (e < 0) return;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -595,7 +653,7 @@ __global__ __launch_bounds__(256) void routed_product_mfma_kernel(const bf16* __
                 if (GATED) {
                     // (gate and up are rounded to the rows' type before the activation, as the plain kernel does)
                     const float gt = bf16_to_f32(f32_to_bf16(acc0[i][j][e4])), up = bf16_to_f32(f32_to_bf16(acc1[i][GATED ? j : 0][e4]));
-                    ((bf16*)out_)[r * n_out + col] = f32_to_bf16(expert_act(gt, act) * up);
+                    ((bf16*)out_)[r * n_out + col] = f32_to_bf16(expert_gated(gt, up, act, p0, p1));
                 } else {
                     ((float*)out_)[r * n_out + col] = acc0[i][j][e4];
                 }
@@ -606,10 +664,10 @@ __global__ __launch_bounds__(256) void routed_product_mfma_kernel(const bf16* __
 // act_rows [cap, ff] bfloat16 and y [cap, hidden] float32 hold sorted rows (see route_sort)
 extern "C" int agave_routed_experts_mfma(const void* x, long ldx, const int* sorted_pair, const int* tile_expert, const void* wg,
                                          const void* wu, const void* wd, void* act_rows, float* y, int TM, int max_tiles, int top,
-                                         int E, int ff, int hidden, int act, int wpacked, hipStream_t stream) {
+                                         int E, int ff, int hidden, int act, int wpacked, float p0, float p1, hipStream_t stream) {
     AGAVE_CHECK(!wpacked || (ff % 32 == 0 && hidden % 32 == 0), "routed_experts_mfma: weights in tile order need sizes that are multiples of 32");
     AGAVE_CHECK(max_tiles > 0 && top > 0 && E > 0 && ff > 0 && hidden > 0 && (TM == 16 || TM == 64), "routed_experts_mfma: bad sizes");
-    AGAVE_CHECK(act >= 0 && act < 4, "routed_experts_mfma: unknown activation %d", act);
+    AGAVE_CHECK((act >= 0 && act < 4) || act == 6, "routed_experts_mfma: unknown activation %d", act);
     AGAVE_CHECK(hidden % 8 == 0 && ff % 8 == 0 && ldx % 8 == 0, "routed_experts_mfma: sizes must be multiples of 8 (hidden %d, ff %d)", hidden, ff);
     AGAVE_CHECK(x && sorted_pair && tile_expert && wg && wu && wd && act_rows && y, "routed_experts_mfma: null buffer");
     AGAVE_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wg % 16) == 0 && ((uintptr_t)wu % 16) == 0 && ((uintptr_t)wd % 16) == 0 &&
@@ -621,14 +679,14 @@ extern "C" int agave_routed_experts_mfma(const void* x, long ldx, const int* sor
     AGAVE_CHECK(g1.y <= 65535 && g2.y <= 65535, "routed_experts_mfma: too many columns for the grid");
     if (TM == 64) {
         routed_product_mfma_kernel<4, 4, true><<<g1, 256, 0, stream>>>((const bf16*)x, ldx, sorted_pair, tile_expert, (const bf16*)wg,
-                                                                    (const bf16*)wu, act_rows, top, ff, hidden, act, wpacked);
+                                                                    (const bf16*)wu, act_rows, top, ff, hidden, act, wpacked, p0, p1);
         routed_product_mfma_kernel<4, 4, false><<<g2, 256, 0, stream>>>((const bf16*)act_rows, ff, sorted_pair, tile_expert, (const bf16*)wd,
-                                                                     nullptr, y, top, hidden, ff, act, wpacked);
+                                                                     nullptr, y, top, hidden, ff, act, wpacked, p0, p1);
     } else {
         routed_product_mfma_kernel<1, 1, true><<<g1, 256, 0, stream>>>((const bf16*)x, ldx, sorted_pair, tile_expert, (const bf16*)wg,
-                                                                    (const bf16*)wu, act_rows, top, ff, hidden, act, wpacked);
+                                                                    (const bf16*)wu, act_rows, top, ff, hidden, act, wpacked, p0, p1);
         routed_product_mfma_kernel<1, 1, false><<<g2, 256, 0, stream>>>((const bf16*)act_rows, ff, sorted_pair, tile_expert, (const bf16*)wd,
-                                                                     nullptr, y, top, hidden, ff, act, wpacked);
+                                                                     nullptr, y, top, hidden, ff, act, wpacked, p0, p1);
     }
     AGAVE_LAUNCH_CHECK("routed_experts_mfma");
     return 0;

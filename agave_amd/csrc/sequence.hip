@@ -28,14 +28,15 @@ __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : __l
 __device__ __forceinline__ float decay_f(float rate, float x) { return __expf(-rate * softplus_f(x)); }
 
 // ------------------------------------------------------------------ short causal convolution
-//   y[t][c] = act(sum_j w[c][j] * u[pos(t) - taps + 1 + j][c]),  zeros before the sequence's start.
+//   y[t][c] = act(bias[c] + sum_j w[c][j] * u[pos(t) - taps + 1 + j][c]),  zeros before the sequence's start
+//   (bias may be null).
 // Inputs older than the step's first token come from state[slot][taps - 1][C], which holds the
 // inputs at positions pos0 - taps + 1 .. pos0 - 1.  fused_update (every sequence brings one token):
 // the thread that owns (sequence, channel) also shifts the state; otherwise conv_state_kernel does
 // it afterwards, when no thread reads the old state any more.
 template <bool SILU>
 __global__ void short_conv_kernel(const float* __restrict__ u, long ldu, const float* __restrict__ w,
-                                  float* __restrict__ y, long ldy, float* __restrict__ state,
+                                  const float* __restrict__ bias, float* __restrict__ y, long ldy, float* __restrict__ state,
                                   const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                   const int* __restrict__ pos0, const int* __restrict__ slots, int C, int taps,
                                   int fused_update) {
@@ -54,7 +55,7 @@ __global__ void short_conv_kernel(const float* __restrict__ u, long ldu, const f
             else in[j] = st_c[(size_t)(r - (p0 - (taps - 1))) * C];
         }
     }
-    float acc = 0.f;
+    float acc = bias ? bias[c] : 0.f;
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS; ++j)
         if (j < taps) acc = fmaf(w[(size_t)c * taps + j], in[j], acc);
@@ -89,7 +90,7 @@ __global__ void conv_state_kernel(const float* __restrict__ u, long ldu, float* 
         if (i < taps - 1) st_c[(size_t)i * C] = keep[i];
 }
 
-extern "C" int agave_short_conv(const float* u, long ldu, const float* w, float* y, long ldy, float* state,
+extern "C" int agave_short_conv(const float* u, long ldu, const float* w, const float* bias, float* y, long ldy, float* state,
                                 const int* tok_seq, const int* tok_pos, const int* cu, const int* pos0,
                                 const int* slots, int n_tokens, int n_seqs, int C, int taps, int silu,
                                 int one_token_each, hipStream_t stream) {
@@ -103,9 +104,9 @@ extern "C" int agave_short_conv(const float* u, long ldu, const float* w, float*
     const int threads = C >= 256 ? 256 : 64;
     const dim3 grid((C + threads - 1) / threads, n_tokens);
     if (silu)
-        short_conv_kernel<true><<<grid, threads, 0, stream>>>(u, ldu, w, y, ldy, state, tok_seq, tok_pos, pos0, slots, C, taps, one_token_each);
+        short_conv_kernel<true><<<grid, threads, 0, stream>>>(u, ldu, w, bias, y, ldy, state, tok_seq, tok_pos, pos0, slots, C, taps, one_token_each);
     else
-        short_conv_kernel<false><<<grid, threads, 0, stream>>>(u, ldu, w, y, ldy, state, tok_seq, tok_pos, pos0, slots, C, taps, one_token_each);
+        short_conv_kernel<false><<<grid, threads, 0, stream>>>(u, ldu, w, bias, y, ldy, state, tok_seq, tok_pos, pos0, slots, C, taps, one_token_each);
     AGAVE_LAUNCH_CHECK("short_conv");
     if (!one_token_each && taps > 1) {
         conv_state_kernel<<<dim3((C + threads - 1) / threads, n_seqs), threads, 0, stream>>>(u, ldu, state, cu, pos0, slots, C, taps);
@@ -535,17 +536,22 @@ extern "C" int agave_talk_attention(int dtype, const float* q, long ldq, const f
 //   delta:   q, k: unit vectors per head (x / sqrt(sum x^2 + unit_eps)), q times dk^-1/2; key head of h is
 //            h / (nh / nkv);  a = exp(-exp(A_log[h]) * softplus(dt[h][d] + dt_bias[h][d]));  beta = sigmoid(b[h])
 //   forget:  q = silu(q);  f = low + (1 - low) sigmoid(f_in + f_bias);  a = f, k = 1 - f
+//   ssd:     one decay per head and token: d = softplus(dt[h] + dt_bias[h]) (exact functions, no clamp),
+//            a = exp(-exp(A_log[h]) d) for every key channel; k = B and q = C of the head's group h / (nh / nkv), as
+//            they come; u = d v; the read-out gets skip[h] v on top
 #define REC_DELTA 0
 #define REC_FORGET 1
+#define REC_SSD 2
 
 struct RecurrenceArgs {
     const float* q; long ldq;          // delta: [N, nkv*dk]; forget: [N, nh*dk]
     const float* k; long ldk;          // delta: keys [N, nkv*dk]; forget: the gate's input [N, nh*dk]
     const float* v; long ldv;          // [N, nh*dv]
-    const float* dt; long lddt;        // delta: [N, nh*dk]
+    const float* dt; long lddt;        // delta: [N, nh*dk]; ssd: [N, nh]
     const float* b; long ldb;          // delta: [N, nh]
-    const float* a_log;                // delta: [nh]
-    const float* dt_bias;              // delta: [nh*dk]
+    const float* a_log;                // delta, ssd: [nh]
+    const float* dt_bias;              // delta: [nh*dk]; ssd: [nh]
+    const float* skip;                 // ssd: [nh]
     const float* low;                  // forget: [nh*dk]
     const float* f_bias;               // forget: [nh*dk] or null
     float* o; long ldo;                // [N, nh*dv]
@@ -554,6 +560,10 @@ struct RecurrenceArgs {
     int nh, nkv, dk, dv;
     float unit_eps;                    // delta: inside the root of the unit vectors
 };
+
+// softplus by the exact functions, for the one step size a head and token has (the state-space form): what it
+// is off by is multiplied into every later state
+__device__ __forceinline__ float softplus_exact(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
 // A lane's R rows of its state column, to and from memory: 16 bytes at a time where the column's
 // length allows (R is a multiple of 4, so a lane's rows start at a multiple of 4 too).
@@ -630,17 +640,19 @@ __global__ __launch_bounds__(512) void gated_recurrence_kernel(RecurrenceArgs A)
     if (!producer) state_load<R>(S, S_g, ds * R, dk, col < dv);
     // ---- producers: what does not change from token to token
     const int pw = wv - 4;
-    const int kvh = MODE == REC_DELTA ? h / (A.nh / A.nkv) : h;
+    const int kvh = MODE == REC_FORGET ? h : h / (A.nh / A.nkv);
     float c0[NE], c1[NE];                                   // delta: dt_bias, -;  forget: lower bound, the gate's bias
     float ea = 0.f;
+    const float skip = MODE == REC_SSD ? A.skip[h] : 0.f;
     if (producer) {
 #pragma unroll
         for (int e = 0; e < NE; ++e) {
             const int d = lane + 64 * e, dd = d < dk ? d : dk - 1;
             if (MODE == REC_DELTA) { c0[e] = A.dt_bias[(size_t)h * dk + dd]; c1[e] = 0.f; }
+            else if (MODE == REC_SSD) { c0[e] = A.dt_bias[h]; c1[e] = 0.f; }
             else { c0[e] = A.low[(size_t)h * dk + dd]; c1[e] = A.f_bias ? A.f_bias[(size_t)h * dk + dd] : 0.f; }
         }
-        if (MODE == REC_DELTA) ea = expf(A.a_log[h]);
+        if (MODE != REC_FORGET) ea = expf(A.a_log[h]);
     }
 
     // what a producer wave has asked for and not yet used: the rows of its tokens of one block
@@ -658,6 +670,10 @@ __global__ __launch_bounds__(512) void gated_recurrence_kernel(RecurrenceArgs A)
                     x0[t][e] = A.q[(size_t)row * A.ldq + (size_t)kvh * dk + dd];
                     x1[t][e] = A.k[(size_t)row * A.ldk + (size_t)kvh * dk + dd];
                     x2[t][e] = A.dt[(size_t)row * A.lddt + (size_t)h * dk + dd];
+                } else if (MODE == REC_SSD) {
+                    x0[t][e] = A.q[(size_t)row * A.ldq + (size_t)kvh * dk + dd];
+                    x1[t][e] = A.k[(size_t)row * A.ldk + (size_t)kvh * dk + dd];
+                    x2[t][e] = 0.f;
                 } else {
                     x0[t][e] = A.q[(size_t)row * A.ldq + (size_t)h * dk + dd];
                     x1[t][e] = A.k[(size_t)row * A.ldk + (size_t)h * dk + dd];
@@ -666,7 +682,7 @@ __global__ __launch_bounds__(512) void gated_recurrence_kernel(RecurrenceArgs A)
             }
             const int c = col0 + (lane < CB ? lane : 0);
             vv[t] = A.v[(size_t)row * A.ldv + (size_t)h * dv + (c < dv ? c : dv - 1)];
-            bb[t] = MODE == REC_DELTA ? A.b[(size_t)row * A.ldb + h] : 0.f;
+            bb[t] = MODE == REC_DELTA ? A.b[(size_t)row * A.ldb + h] : (MODE == REC_SSD ? A.dt[(size_t)row * A.lddt + h] : 0.f);
         }
     };
     auto make = [&](int blk, int buf) {
@@ -687,6 +703,11 @@ __global__ __launch_bounds__(512) void gated_recurrence_kernel(RecurrenceArgs A)
                 qi = 1.0f / sqrtf(qq + A.unit_eps) / sqrtf((float)dk);
                 ki = 1.0f / sqrtf(kk + A.unit_eps);
             }
+            float step = 0.f, step_decay = 1.f;             // ssd: the token's step size and what it leaves of the state
+            if (MODE == REC_SSD) {
+                step = softplus_exact(bb[t] + c0[0]);
+                step_decay = expf(-ea * step);
+            }
             float kq = 0.f;
 #pragma unroll
             for (int e = 0; e < NE; ++e) {
@@ -697,6 +718,10 @@ __global__ __launch_bounds__(512) void gated_recurrence_kernel(RecurrenceArgs A)
                         a = decay_f(ea, x2[t][e] + c0[e]);
                         kx = x1[t][e] * ki;
                         qx = x0[t][e] * qi;
+                    } else if (MODE == REC_SSD) {
+                        a = step_decay;
+                        kx = x1[t][e];
+                        qx = x0[t][e];
                     } else {
                         const float f = c0[e] + (1.f - c0[e]) * sigmoid_f(x1[t][e] + c1[e]);
                         a = f;
@@ -710,7 +735,7 @@ __global__ __launch_bounds__(512) void gated_recurrence_kernel(RecurrenceArgs A)
             kq = wave_sum(kq);
             if (lane < CB) sv[buf][tt][lane] = real ? vv[t] : 0.f;
             if (lane == 0) {
-                sbeta[buf][tt] = (MODE == REC_DELTA && real) ? sigmoid_f(bb[t]) : (real ? 1.f : 0.f);
+                sbeta[buf][tt] = (MODE == REC_DELTA && real) ? sigmoid_f(bb[t]) : (MODE == REC_SSD ? step : (real ? 1.f : 0.f));
                 skq[buf][tt] = kq;
             }
         }
@@ -751,9 +776,12 @@ __global__ __launch_bounds__(512) void gated_recurrence_kernel(RecurrenceArgs A)
         } else {
             dq = lanes_sum<DS>(dq);
         }
+        const float v_in = u;
+        if (MODE == REC_SSD) u *= sbeta[buf][tt];
 #pragma unroll
         for (int i = 0; i < R; ++i) S[i] = fmaf(kreg[i], u, S[i]);
-        const float o = fmaf(u, skq[buf][tt], dq);
+        float o = fmaf(u, skq[buf][tt], dq);
+        if (MODE == REC_SSD) o = fmaf(skip, v_in, o);
         if (ds == 0 && col < dv) A.o[(size_t)(tb + tt) * A.ldo + (size_t)h * dv + col] = o;
     };
     auto consume = [&](int blk, int buf) {
@@ -805,7 +833,7 @@ __global__ __launch_bounds__(256) void gated_recurrence_step_kernel(RecurrenceAr
     float* S_g = A.state + (((size_t)A.slots[s] * A.nh + h) * dv + (col < dv ? col : 0)) * dk;
     float S[R];
     state_load<R>(S, S_g, ds * R, dk, col < dv);
-    const int kvh = MODE == REC_DELTA ? h / (A.nh / A.nkv) : h;
+    const int kvh = MODE == REC_FORGET ? h : h / (A.nh / A.nkv);
     float x0[NE], x1[NE], x2[NE], c0[NE], c1[NE];
 #pragma unroll
     for (int e = 0; e < NE; ++e) {                          // every load first
@@ -816,6 +844,11 @@ __global__ __launch_bounds__(256) void gated_recurrence_step_kernel(RecurrenceAr
             x2[e] = A.dt[row * A.lddt + (size_t)h * dk + dd];
             c0[e] = A.dt_bias[(size_t)h * dk + dd];
             c1[e] = 0.f;
+        } else if (MODE == REC_SSD) {
+            x0[e] = A.q[row * A.ldq + (size_t)kvh * dk + dd];
+            x1[e] = A.k[row * A.ldk + (size_t)kvh * dk + dd];
+            x2[e] = 0.f;
+            c0[e] = c1[e] = 0.f;
         } else {
             x0[e] = A.q[row * A.ldq + (size_t)h * dk + dd];
             x1[e] = A.k[row * A.ldk + (size_t)h * dk + dd];
@@ -829,6 +862,14 @@ __global__ __launch_bounds__(256) void gated_recurrence_step_kernel(RecurrenceAr
     if (MODE == REC_DELTA) {
         beta = sigmoid_f(A.b[row * A.ldb + h]);
         ea = expf(A.a_log[h]);
+    }
+    float step = 0.f, step_decay = 1.f, skip = 0.f;
+    const float v_in = u;
+    if (MODE == REC_SSD) {
+        step = softplus_exact(A.dt[row * A.lddt + h] + A.dt_bias[h]);
+        step_decay = expf(-expf(A.a_log[h]) * step);
+        skip = A.skip[h];
+        u *= step;
     }
     float qi = 1.f, ki = 1.f;
     if (MODE == REC_DELTA) {
@@ -851,6 +892,10 @@ __global__ __launch_bounds__(256) void gated_recurrence_step_kernel(RecurrenceAr
                 a = decay_f(ea, x2[e] + c0[e]);
                 kx = x1[e] * ki;
                 qx = x0[e] * qi;
+            } else if (MODE == REC_SSD) {
+                a = step_decay;
+                kx = x1[e];
+                qx = x0[e];
             } else {
                 const float f = c0[e] + (1.f - c0[e]) * sigmoid_f(x1[e] + c1[e]);
                 a = f;
@@ -878,7 +923,7 @@ __global__ __launch_bounds__(256) void gated_recurrence_step_kernel(RecurrenceAr
 #pragma unroll
     for (int i = 0; i < R; ++i) S[i] = fmaf(kreg[i], u, S[i]);
     state_store<R>(S, S_g, ds * R, dk, col < dv);
-    if (ds == 0 && col < dv) A.o[row * A.ldo + (size_t)h * dv + col] = fmaf(u, kq, dq);
+    if (ds == 0 && col < dv) A.o[row * A.ldo + (size_t)h * dv + col] = fmaf(u, kq, dq) + skip * v_in;
 }
 
 template <int MODE>
@@ -909,10 +954,10 @@ static int launch_recurrence(const RecurrenceArgs& A, int n_seqs, hipStream_t st
 
 extern "C" int agave_gated_recurrence(int mode, const float* q, long ldq, const float* k, long ldk, const float* v, long ldv,
                                       const float* dt, long lddt, const float* b, long ldb, const float* a_log,
-                                      const float* dt_bias, const float* low, const float* f_bias, float* o, long ldo,
+                                      const float* dt_bias, const float* low, const float* f_bias, const float* skip, float* o, long ldo,
                                       float* state, const int* cu, const int* slots, int n_seqs, int nh, int nkv, int dk,
                                       int dv, float unit_eps, int one_token_each, hipStream_t stream) {
-    AGAVE_CHECK(mode == REC_DELTA || mode == REC_FORGET, "gated_recurrence: unknown mode %d", mode);
+    AGAVE_CHECK(mode == REC_DELTA || mode == REC_FORGET || mode == REC_SSD, "gated_recurrence: unknown mode %d", mode);
     AGAVE_CHECK(n_seqs >= 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "gated_recurrence: bad sizes B=%d nh=%d nkv=%d dk=%d dv=%d", n_seqs, nh, nkv, dk, dv);
     AGAVE_CHECK(dk <= 256, "gated_recurrence: %d key channels a head (up to 256 are supported)", dk);
     AGAVE_CHECK(nh % nkv == 0, "gated_recurrence: %d heads are not a multiple of %d key heads", nh, nkv);
@@ -922,14 +967,20 @@ extern "C" int agave_gated_recurrence(int mode, const float* q, long ldq, const 
     if (mode == REC_DELTA) {
         AGAVE_CHECK(dt && b && a_log && dt_bias, "gated_recurrence: the delta rule needs dt, b, A_log and dt_bias");
         AGAVE_CHECK(ldq >= (long)nkv * dk && ldk >= (long)nkv * dk && lddt >= (long)nh * dk && ldb >= nh, "gated_recurrence: a row stride is too small");
+    } else if (mode == REC_SSD) {
+        AGAVE_CHECK(dt && a_log && dt_bias && skip, "gated_recurrence: the state-space form needs dt, A_log, dt_bias and the skip weights");
+        AGAVE_CHECK(ldq >= (long)nkv * dk && ldk >= (long)nkv * dk && lddt >= nh, "gated_recurrence: a row stride is too small");
     } else {
         AGAVE_CHECK(low, "gated_recurrence: the forget gate needs its lower bound");
         AGAVE_CHECK(nkv == nh && ldq >= (long)nh * dk && ldk >= (long)nh * dk, "gated_recurrence: the forget-gate form has a gate per head");
     }
     if (n_seqs == 0) return 0;
-    RecurrenceArgs A{q, ldq, k, ldk, v, ldv, dt, lddt, b, ldb, a_log, dt_bias, low, f_bias, o, ldo, state, cu, slots, nh, nkv, dk, dv, unit_eps};
-    if (one_token_each)                                     // the host vouches that every sequence brings one token
+    RecurrenceArgs A{q, ldq, k, ldk, v, ldv, dt, lddt, b, ldb, a_log, dt_bias, skip, low, f_bias, o, ldo, state, cu, slots, nh, nkv, dk, dv, unit_eps};
+    if (one_token_each) {                                   // the host vouches that every sequence brings one token
+        if (mode == REC_SSD) return launch_recurrence_step<REC_SSD>(A, n_seqs, stream);
         return mode == REC_DELTA ? launch_recurrence_step<REC_DELTA>(A, n_seqs, stream) : launch_recurrence_step<REC_FORGET>(A, n_seqs, stream);
+    }
+    if (mode == REC_SSD) return launch_recurrence<REC_SSD>(A, n_seqs, stream);
     return mode == REC_DELTA ? launch_recurrence<REC_DELTA>(A, n_seqs, stream) : launch_recurrence<REC_FORGET>(A, n_seqs, stream);
 }
 
@@ -965,6 +1016,45 @@ extern "C" int agave_head_norm_gate(int dtype, const float* o, long ldo_in, cons
     else
         AGAVE_CHECK(false, "head_norm_gate: unknown dtype %d", dtype);
     AGAVE_LAUNCH_CHECK("head_norm_gate");
+    return 0;
+}
+
+// ------------------------------------------------------------------ a gate, then a norm in equal parts of the row
+//   g = y * silu(z);  out = g / sqrt(mean over the part (g^2) + eps) * w     (a wave per (token, part); w is [parts * size])
+template <typename T>
+__global__ __launch_bounds__(64) void gated_group_norm_kernel(const float* __restrict__ y, long ldy, const float* __restrict__ z,
+                                                              long ldz, const float* __restrict__ w, T* __restrict__ out, long ldo,
+                                                              int parts, int size, float eps) {
+    const int t = blockIdx.x / parts, g = blockIdx.x % parts, lane = threadIdx.x;
+    const float* yr = y + (size_t)t * ldy + (size_t)g * size;
+    const float* zr = z + (size_t)t * ldz + (size_t)g * size;
+    float ss = 0.f;
+    for (int e = lane; e < size; e += 64) {
+        const float zv = zr[e], v = yr[e] * (zv / (1.0f + expf(-zv)));
+        ss = fmaf(v, v, ss);
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)size + eps);
+    for (int e = lane; e < size; e += 64) {
+        const float zv = zr[e], v = yr[e] * (zv / (1.0f + expf(-zv)));
+        st(out + (size_t)t * ldo + (size_t)g * size + e, v * inv * w[(size_t)g * size + e]);
+    }
+}
+
+extern "C" int agave_gated_group_norm(int dtype, const float* y, long ldy, const float* z, long ldz, const float* w, void* out,
+                                      long ldo, int N, int parts, int size, float eps, hipStream_t stream) {
+    AGAVE_CHECK(N >= 0 && parts > 0 && size > 0, "gated_group_norm: bad sizes N=%d parts=%d size=%d", N, parts, size);
+    const long width = (long)parts * size;
+    AGAVE_CHECK(y && z && w && out && ldy >= width && ldz >= width && ldo >= width, "gated_group_norm: bad buffers");
+    AGAVE_CHECK((long)N * parts < 2147483647L, "gated_group_norm: too many rows");
+    if (N == 0) return 0;
+    if (dtype == AGAVE_F32)
+        gated_group_norm_kernel<float><<<N * parts, 64, 0, stream>>>(y, ldy, z, ldz, w, (float*)out, ldo, parts, size, eps);
+    else if (dtype == AGAVE_BF16)
+        gated_group_norm_kernel<bf16><<<N * parts, 64, 0, stream>>>(y, ldy, z, ldz, w, (bf16*)out, ldo, parts, size, eps);
+    else
+        AGAVE_CHECK(false, "gated_group_norm: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("gated_group_norm");
     return 0;
 }
 

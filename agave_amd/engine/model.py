@@ -22,6 +22,8 @@ from ..weights.loader import TensorNeed
 def tensor_needs(spec: ModelSpec) -> List[TensorNeed]:
     """Every tensor the model reads, in a fixed order (embedding, layers, final norm, head)."""
     needs = [TensorNeed(spec.embed_weight, (spec.vocab_size, spec.hidden))]
+    if spec.embed_norm is not None:
+        needs += lookup("norm", spec.embed_norm.kind).tensor_needs(spec.embed_norm)
     for layer in spec.layers:
         needs += lookup("block", layer.kind).tensor_needs(layer)
     if spec.final_norm is not None:
@@ -40,6 +42,8 @@ class Model:
         if table.dtype != keep:
             table = table.to(keep)
         self.embed_table: Optional[torch.Tensor] = table.to(env.device).contiguous()
+        self.embed_norm = (lookup("norm", spec.embed_norm.kind)(spec.embed_norm, weights, env)
+                           if spec.embed_norm is not None else None)
         self.blocks = [lookup("block", layer.kind)(layer, weights, env) for layer in spec.layers]
         self.final_norm = (lookup("norm", spec.final_norm.kind)(spec.final_norm, weights, env)
                            if spec.final_norm is not None else None)
@@ -87,7 +91,7 @@ class Model:
 
     def weight_bytes(self) -> int:
         """Bytes of all weights on the device, shared tensors counted once."""
-        parts = [self.embed_table, self.blocks, self.final_norm, self.head]
+        parts = [self.embed_table, self.embed_norm, self.blocks, self.final_norm, self.head]
         return sum(t.numel() * t.element_size() for t in part_tensors(parts))
 
     # ------------------------------------------------------------------ one step
@@ -96,11 +100,18 @@ class Model:
         ws = self.env.workspace
         n = step.n_tokens
         h = ws.get("residual", n, self.spec.hidden, torch.float32)
-        if self.embed_table is not None:
-            kernels.embed_scale(step.tokens, self.embed_table, self.spec.embed_scale, h)
-        else:
-            gemm_mfma.embed_scale_packed(step.tokens, self.head.packed, self.spec.embed_scale, h, self.spec.vocab_size)
         pending = None
+        rows = h
+        if self.embed_norm is not None:
+            # the stream starts at zero and the embedding rows are its first branch, added through their norm by
+            # whoever adds a branch next (one 32-bit slice: the rows are not rounded on the way)
+            rows = ws.get3("embedded", 1, n, self.spec.hidden, torch.float32)[0]
+            pending = (rows.view(1, n, self.spec.hidden), self.embed_norm)
+            h.zero_()
+        if self.embed_table is not None:
+            kernels.embed_scale(step.tokens, self.embed_table, self.spec.embed_scale, rows)
+        else:
+            gemm_mfma.embed_scale_packed(step.tokens, self.head.packed, self.spec.embed_scale, rows, self.spec.vocab_size)
         for entry in self.spec.order:
             pending = self.blocks[entry.layer].forward(h, pending, step, entry.memory, entry.writes)
         if step.n_want == 0:

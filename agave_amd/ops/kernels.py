@@ -26,7 +26,7 @@ _SIGNATURES = {
         "agave_qk_norm_rope_kv": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F,
                                   _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
         "agave_geglu": [_I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
-        "agave_gated_act": [_I, _I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
+        "agave_gated_act": [_I, _I, _F, _F, _P, _L, _P, _L, _P, _L, _I, _I, _P],
         "agave_unary_act": [_I, _I, _F, _F, _P, _L, _P, _L, _I, _I, _P],
         "agave_cast": [_I, _P, _I, _P, _L, _P],
         "agave_add_bias": [_I, _P, _L, _P, _I, _I, _P],
@@ -293,11 +293,14 @@ def _check_table(table: torch.Tensor, base: torch.Tensor, tok_seq: Optional[torc
 
 
 # The activations of a gated feed-forward that the elementwise kernel knows, by the number it knows them by.
-GATE_ACTIVATIONS = {"gelu_tanh": 0, "silu": 1, "gelu": 2, "relu": 3}
+# ``swish_clamped`` has two numbers of its own: g = min(gate, p0), u = clamp(up, -p0, p0), out = g sigmoid(p1 g) (u + 1).
+GATE_ACTIVATIONS = {"gelu_tanh": 0, "silu": 1, "gelu": 2, "relu": 3, "swish_clamped": 6}
 
 
-def gated_act(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor, activation: str = "gelu_tanh") -> None:
-    """out = act(gate) * up, row by row; ``activation`` is one of ``GATE_ACTIVATIONS``."""
+def gated_act(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor, activation: str = "gelu_tanh", p0: float = 0.0,
+              p1: float = 1.0) -> None:
+    """out = act(gate) * up, row by row; ``activation`` is one of ``GATE_ACTIVATIONS`` (``p0``, ``p1``: the numbers of
+    ``swish_clamped``)."""
     _dev(gate, up, out)
     try:
         act = GATE_ACTIVATIONS[activation]
@@ -307,12 +310,12 @@ def gated_act(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor, activatio
     if gate.shape != up.shape or gate.shape != out.shape or not (gate.dtype == up.dtype == out.dtype):
         raise ValueError("gated_act: gate, up and out must agree in shape and dtype")
     n, ff = gate.shape
-    library.call(lib("elementwise"), "agave_gated_act", dt(gate), act, ptr(gate), ldg, ptr(up), ldu, ptr(out), ldo, n, ff,
+    library.call(lib("elementwise"), "agave_gated_act", dt(gate), act, float(p0), float(p1), ptr(gate), ldg, ptr(up), ldu, ptr(out), ldo, n, ff,
                  stream())
 
 
 # The activations of a feed-forward without a gate: the gate's, xIELU with two learned numbers, and the square of ReLU.
-UNARY_ACTIVATIONS = dict(GATE_ACTIVATIONS, xielu=4, relu2=5)
+UNARY_ACTIVATIONS = dict({k: v for k, v in GATE_ACTIVATIONS.items() if v < 4}, xielu=4, relu2=5)
 
 
 def unary_act(x: torch.Tensor, out: torch.Tensor, activation: str, p0: float = 0.0, p1: float = 0.0) -> None:

@@ -13,11 +13,11 @@ MAX_OUTPUTS = 1024
 
 kernels.register_signatures(LIBRARY, {
     "agave_route_topk": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _F, _P, _P, _P],
-    "agave_routed_experts_plain": [_I, _P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
-    "agave_route_rows": [_I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P, _P],
+    "agave_routed_experts_plain": [_I, _P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _P],
+    "agave_route_rows": [_I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P, _I, _I, _P, _P],
     "agave_route_sort": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
-    "agave_routed_experts_mfma": [_P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
-    "agave_routed_combine": [_I, _P, _P, _P, _P, _P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _P],
+    "agave_routed_experts_mfma": [_P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
+    "agave_routed_combine": [_I, _P, _P, _P, _P, _P, _L, _P, _L, _P, _P, _L, _I, _I, _I, _I, _P],
 })
 
 
@@ -45,7 +45,7 @@ def route_topk(logits: torch.Tensor, correction: Optional[torch.Tensor], scratch
 
 
 def experts_plain(x: torch.Tensor, choice: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
-                  act_rows: torch.Tensor, y: torch.Tensor, top: int, activation: int) -> None:
+                  act_rows: torch.Tensor, y: torch.Tensor, top: int, activation: int, p0: float = 0.0, p1: float = 1.0) -> None:
     """y[p] = W_down[e] (act(W_gate[e] x_t) * (W_up[e] x_t)) for every pair p = t * top + slot whose choice e is an
     expert with weights (e < E); rows of other pairs are left alone.  ``y`` is float32 [N * top, hidden]."""
     _dev(x, choice, w_gate, w_up, w_down, act_rows, y)
@@ -63,14 +63,17 @@ def experts_plain(x: torch.Tensor, choice: torch.Tensor, w_gate: torch.Tensor, w
     if y.dtype != torch.float32 or not y.is_contiguous() or y.shape != (n * top, hidden):
         raise ValueError(f"experts: y must be float32 [{n * top}, {hidden}]")
     library.call(_lib(), "agave_routed_experts_plain", dt(x), ptr(x), ldx, ptr(choice), ptr(w_gate), ptr(w_up), ptr(w_down),
-                 ptr(act_rows), ptr(y), n, top, e, ff, hidden, activation, stream())
+                 ptr(act_rows), ptr(y), n, top, e, ff, hidden, activation, float(p0), float(p1), stream())
 
 
 def combine(y: Optional[torch.Tensor], place: Optional[torch.Tensor], choice: torch.Tensor, weight: torch.Tensor,
-            x: torch.Tensor, shared: Optional[torch.Tensor], out: torch.Tensor, top: int, n_experts: int) -> None:
+            x: torch.Tensor, shared: Optional[torch.Tensor], out: torch.Tensor, top: int, n_experts: int,
+            shared_gate: Optional[torch.Tensor] = None) -> None:
     """out[t] = sum over the token's pairs of weight * (the pair's expert row of ``y``, or ``x[t]`` itself where the
-    choice is an identity expert, e >= n_experts) + shared[t]."""
-    _dev(y, place, choice, weight, x, shared, out)
+    choice is an identity expert, e >= n_experts) + shared[t], the latter times ``sigmoid(shared_gate[t])`` where a
+    float32 logit per token is given."""
+    _dev(y, place, choice, weight, x, shared, out, shared_gate)
+    _f32vec(shared_gate, "shared_gate", x.shape[0])
     n, hidden = x.shape
     ldx, ldo = _rows(x, "x"), _rows(out, "out")
     if out.shape != x.shape or out.dtype != x.dtype:
@@ -85,7 +88,7 @@ def combine(y: Optional[torch.Tensor], place: Optional[torch.Tensor], choice: to
     _i32(choice, "choice", n * top)
     _i32(place, "place", n * top)
     library.call(_lib(), "agave_routed_combine", dt(x), ptr(y), ptr(place), ptr(choice), ptr(weight), ptr(x), ldx, ptr(shared),
-                 lds, ptr(out), ldo, n, top, n_experts, hidden, stream())
+                 lds, ptr(shared_gate) if shared is not None else None, ptr(out), ldo, n, top, n_experts, hidden, stream())
 
 
 def tile_plan(n_pairs: int, n_experts: int):
@@ -119,7 +122,7 @@ def route_sort(choice: torch.Tensor, n_experts: int, tm: int, tiles: int, place:
 
 def experts_mfma(x: torch.Tensor, sorted_pair: torch.Tensor, tile_expert: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
                  w_down: torch.Tensor, act_rows: torch.Tensor, y: torch.Tensor, tm: int, tiles: int, top: int, activation: int,
-                 tile_order: bool = False) -> None:
+                 tile_order: bool = False, p0: float = 0.0, p1: float = 1.0) -> None:
     """The experts' products over the sorted rows on the matrix cores: ``act_rows`` [tiles * tm, ff] bfloat16 and
     ``y`` [tiles * tm, hidden] float32 receive sorted rows (padding rows hold nothing of use).  ``tile_order``: the
     weights were rearranged by :func:`pack_expert_weights` (same shapes)."""
@@ -142,25 +145,39 @@ def experts_mfma(x: torch.Tensor, sorted_pair: torch.Tensor, tile_expert: torch.
     _i32(tile_expert, "tile_expert", tiles)
     library.call(_lib(), "agave_routed_experts_mfma", ptr(x), x.stride(0), ptr(sorted_pair), ptr(tile_expert), ptr(w_gate),
                  ptr(w_up), ptr(w_down), ptr(act_rows), ptr(y), tm, tiles, top, e, ff, hidden, activation,
-                 1 if tile_order else 0, stream())
+                 1 if tile_order else 0, float(p0), float(p1), stream())
 
 
 def route_rows(x: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int, top: int,
-               scale: float, choice: torch.Tensor, weight: torch.Tensor) -> None:
+               scale: float, choice: torch.Tensor, weight: torch.Tensor, softmax_top: bool = False,
+               extra_out: Optional[torch.Tensor] = None) -> None:
     """The router's 32-bit product ``x router^T`` and :func:`route_topk`'s choice in one kernel (the logits never
-    leave the compute unit).  ``router`` is float32 [R, width]; ``x`` [N, width] in either element type."""
-    _dev(x, router, correction, choice, weight)
+    leave the compute unit).  ``router`` is float32 [R, width]; ``x`` [N, width] in either element type.
+    ``softmax_top``: the ``top`` largest logits + ``correction`` are chosen (the lower index among equals) and their
+    weights are the softmax over the chosen alone, times ``scale`` (no groups, ``top`` <= 64).  ``extra_out``
+    (float32 [N, extra]): the router matrix has ``extra`` further rows behind its outputs, whose products with
+    the rows are left there as they are."""
+    _dev(x, router, correction, choice, weight, extra_out)
     n, k = x.shape
     ldx = _rows(x, "x")
     if router.dtype != torch.float32 or router.dim() != 2 or router.shape[1] != k or not router.is_contiguous():
         raise ValueError(f"route_rows: the router must be contiguous float32 [outputs, {k}]")
-    r = router.shape[0]
+    extra = 0
+    if extra_out is not None:
+        if extra_out.dtype != torch.float32 or extra_out.dim() != 2 or extra_out.shape[0] != n or not extra_out.is_contiguous():
+            raise ValueError(f"route_rows: extra_out must be contiguous float32 [{n}, extra]")
+        extra = extra_out.shape[1]
+    r = router.shape[0] - extra
+    if r < 1:
+        raise ValueError("route_rows: the router has no outputs")
+    if softmax_top and (groups != 1 or keep != 1 or top > 64):
+        raise ValueError("route_rows: the softmax over the chosen logits takes no groups and at most 64 chosen")
     _f32vec(correction, "correction", r)
     _i32(choice, "choice", n * top)
     if weight.dtype != torch.float32 or not weight.is_contiguous() or weight.numel() < n * top:
         raise ValueError("route_rows: weight must be contiguous float32 [N, top]")
     library.call(_lib(), "agave_route_rows", dt(x), ptr(x), ldx, ptr(router), ptr(correction), n, k, r, groups, keep, top,
-                 float(scale), ptr(choice), ptr(weight), stream())
+                 float(scale), ptr(choice), ptr(weight), 1 if softmax_top else 0, extra, ptr(extra_out), stream())
 
 
 def pack_expert_weights(w: torch.Tensor) -> torch.Tensor:

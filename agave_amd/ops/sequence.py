@@ -18,19 +18,20 @@ from .kernels import _P, _I, _L, _F, _dev, _f32vec, _i32, dt, ptr, stream
 LIBRARY = "sequence"
 
 kernels.register_signatures(LIBRARY, {
-    "agave_short_conv": [_P, _L, _P, _P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "agave_short_conv": [_P, _L, _P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "agave_head_norm_rope_rows": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _I, _I, _P, _I, _I, _P, _P,
                                   _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "agave_talk_attention": [_I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I,
                              _F, _I, _F, _P, _I, _P],
-    "agave_gated_recurrence": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _L, _P, _P, _P,
+    "agave_gated_recurrence": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P,
                                _I, _I, _I, _I, _I, _F, _I, _P],
+    "agave_gated_group_norm": [_I, _P, _L, _P, _L, _P, _P, _L, _I, _I, _I, _F, _P],
     "agave_head_norm_gate": [_I, _P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _F, _F, _P],
     "agave_scaled_sum": [_I, _P, _L, _F, _P, _L, _F, _P, _L, _I, _I, _P],
 })
 
 MAX_TAPS = 8
-DELTA, FORGET = 0, 1
+DELTA, FORGET, SSD = 0, 1, 2
 
 
 def _lib():
@@ -44,10 +45,12 @@ def _f32rows(t: torch.Tensor, what: str, n: int, cols: int) -> int:
     return t.stride(0)
 
 
-def short_conv(u: torch.Tensor, weight: torch.Tensor, y: torch.Tensor, state: torch.Tensor, step, silu: bool) -> None:
-    """y[t, c] = act(sum_j weight[c, j] * u[t - taps + 1 + j, c]) along each sequence, zeros before its
+def short_conv(u: torch.Tensor, weight: torch.Tensor, y: torch.Tensor, state: torch.Tensor, step, silu: bool,
+               bias: Optional[torch.Tensor] = None) -> None:
+    """y[t, c] = act(bias[c] + sum_j weight[c, j] * u[t - taps + 1 + j, c]) along each sequence, zeros before its
     start; ``state`` [slots, taps - 1, C] holds each sequence's last inputs and is advanced."""
-    _dev(u, weight, y, state)
+    _dev(u, weight, y, state, bias)
+    _f32vec(bias, "conv bias", weight.shape[0])
     n = step.n_tokens
     c, taps = weight.shape
     ldu, ldy = _f32rows(u, "conv input", n, c), _f32rows(y, "conv output", n, c)
@@ -59,7 +62,7 @@ def short_conv(u: torch.Tensor, weight: torch.Tensor, y: torch.Tensor, state: to
         raise ValueError(f"short_conv: state must be float32 [slots, {taps - 1}, {c}], got {tuple(state.shape)}")
     if max(step.slots) >= state.shape[0]:
         raise ValueError("short_conv: a slot lies outside the state")
-    library.call(_lib(), "agave_short_conv", ptr(u), ldu, ptr(weight), ptr(y), ldy, ptr(state), ptr(step.tok_seq),
+    library.call(_lib(), "agave_short_conv", ptr(u), ldu, ptr(weight), ptr(bias), ptr(y), ldy, ptr(state), ptr(step.tok_seq),
                  ptr(step.tok_pos), ptr(step.cu_dev), ptr(step.pos0_dev), ptr(step.slots_dev), n, step.n_seqs, c, taps,
                  1 if silu else 0, 1 if step.is_decode else 0, stream())
 
@@ -150,7 +153,7 @@ def gated_recurrence(mode: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
                      dt_in: Optional[torch.Tensor] = None, beta: Optional[torch.Tensor] = None,
                      a_log: Optional[torch.Tensor] = None, dt_bias: Optional[torch.Tensor] = None,
                      lower: Optional[torch.Tensor] = None, f_bias: Optional[torch.Tensor] = None,
-                     unit_eps: float = 1e-6) -> None:
+                     skip: Optional[torch.Tensor] = None, unit_eps: float = 1e-6) -> None:
     """Advance ``state`` [slots, heads, dv, dk] (a column of S lies together) over the step's tokens, sequence by sequence, and
     write each token's read-out to ``out`` [N, heads * dv] (float32).
 
@@ -158,10 +161,12 @@ def gated_recurrence(mode: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
     a = exp(-exp(a_log[h]) * softplus(dt_in + dt_bias)) per head and key channel; beta = sigmoid(beta);
     S <- diag(a) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
     ``FORGET``: q = silu(q), f = lower + (1 - lower) sigmoid(k + f_bias) with k the gate's input;
-    S <- diag(f) S + (1 - f) v^T;  o = S^T q."""
-    _dev(q, k, v, out, state, dt_in, beta, a_log, dt_bias, lower, f_bias)
+    S <- diag(f) S + (1 - f) v^T;  o = S^T q.
+    ``SSD``:    q, k [N, n_kv * dk] as they come (head h reads group h // (heads / n_kv)); one step size per head
+    and token, d = softplus(dt_in[t, h] + dt_bias[h]);  S <- exp(-exp(a_log[h]) d) S + d k v^T;  o = S^T q + skip[h] v."""
+    _dev(q, k, v, out, state, dt_in, beta, a_log, dt_bias, lower, f_bias, skip)
     n = step.n_tokens
-    kw = (n_kv if mode == DELTA else n_heads) * dk
+    kw = (n_heads if mode == FORGET else n_kv) * dk
     ldq, ldk = _f32rows(q, "q", n, kw), _f32rows(k, "k", n, kw)
     ldv, ldo = _f32rows(v, "v", n, n_heads * dv), _f32rows(out, "out", n, n_heads * dv)
     if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (n_heads, dv, dk):
@@ -175,6 +180,13 @@ def gated_recurrence(mode: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
         _f32vec(dt_bias, "dt_bias", n_heads * dk)
         if a_log is None or dt_bias is None:
             raise ValueError("gated_recurrence: the delta rule needs a_log and dt_bias")
+    elif mode == SSD:
+        lddt = _f32rows(dt_in, "dt", n, n_heads)
+        _f32vec(a_log, "a_log", n_heads)
+        _f32vec(dt_bias, "dt_bias", n_heads)
+        _f32vec(skip, "skip", n_heads)
+        if a_log is None or dt_bias is None or skip is None:
+            raise ValueError("gated_recurrence: the state-space form needs a_log, dt_bias and skip")
     elif mode == FORGET:
         _f32vec(lower, "lower", n_heads * dk)
         _f32vec(f_bias, "f_bias", n_heads * dk)
@@ -183,8 +195,8 @@ def gated_recurrence(mode: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
     else:
         raise ValueError(f"gated_recurrence: unknown mode {mode}")
     library.call(_lib(), "agave_gated_recurrence", mode, ptr(q), ldq, ptr(k), ldk, ptr(v), ldv, ptr(dt_in), lddt, ptr(beta),
-                 ldb, ptr(a_log), ptr(dt_bias), ptr(lower), ptr(f_bias), ptr(out), ldo, ptr(state), ptr(step.cu_dev),
-                 ptr(step.slots_dev), step.n_seqs, n_heads, n_kv if mode == DELTA else n_heads, dk, dv, float(unit_eps),
+                 ldb, ptr(a_log), ptr(dt_bias), ptr(lower), ptr(f_bias), ptr(skip), ptr(out), ldo, ptr(state), ptr(step.cu_dev),
+                 ptr(step.slots_dev), step.n_seqs, n_heads, n_heads if mode == FORGET else n_kv, dk, dv, float(unit_eps),
                  1 if (step.is_decode and step.n_tokens == step.n_seqs) else 0, stream())
 
 
@@ -202,6 +214,22 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: Optional[torch.T
     _f32vec(weight, "weight", dv)
     library.call(_lib(), "agave_head_norm_gate", dt(out), ptr(o), ldi, ptr(weight), ptr(gate), ldg, ptr(out), ldo, n,
                  n_heads, dv, float(eps), float(out_scale), stream())
+
+
+def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, parts: int, eps: float) -> None:
+    """g = y * silu(z); every one of the ``parts`` equal parts of a row of g is divided by its own root mean square
+    (eps inside the root) and multiplied by ``weight`` [width]; ``y``, ``z`` float32 [N, width], ``out`` in its own dtype."""
+    _dev(y, z, weight, out)
+    n, width = y.shape
+    if width % parts:
+        raise ValueError(f"gated_group_norm: rows of {width} do not split into {parts} equal parts")
+    ldy, ldz = _f32rows(y, "y", n, width), _f32rows(z, "z", n, width)
+    ldo = kernels._rows(out, "out")
+    if tuple(out.shape) != (n, width):
+        raise ValueError(f"gated_group_norm: out must be [{n}, {width}], got {tuple(out.shape)}")
+    _f32vec(weight, "weight", width)
+    library.call(_lib(), "agave_gated_group_norm", dt(out), ptr(y), ldy, ptr(z), ldz, ptr(weight), ptr(out), ldo, n, parts,
+                 width // parts, float(eps), stream())
 
 
 def scaled_sum(a: torch.Tensor, sa: float, b: torch.Tensor, sb: float, out: torch.Tensor) -> None:

@@ -4,7 +4,12 @@
 
     h += post_mixer_norm(mixer(pre_mixer_norm(h)));  h += post_ffn_norm(ffn(pre_ffn_norm(h)))
 
-``prenorm`` is the same without the two post norms.  A block never adds its last branch
+``prenorm`` is the same without the two post norms.  ``postnorm`` has no norm in front of a sublayer: the
+sublayers read the stream itself, rounded to the activations' type,
+
+    h += post_mixer_norm(mixer(h));  h += post_ffn_norm(ffn(h))
+
+A block never adds its last branch
 itself: it returns it as *pending* ``(branch, norm | None)``, and whoever runs next (the
 next block's first norm, or the model's end) hands it to the norm that comes next
 (``norm.add_and_norm``), which adds it and computes itself, in one kernel where the kinds of
@@ -108,5 +113,44 @@ class PreNormBlock(SandwichBlock):
     post_norms = False
 
 
+class PostNormBlock(SandwichBlock):
+    """No norm in front of a sublayer, one behind it.  The pending branch is added and the stream's rows are handed
+    to the sublayer as they are (one kernel, as with a norm in front)."""
+
+    def __init__(self, spec: LayerSpec, weights, env: BuildEnv):
+        self.spec, self.env = spec, env
+
+        def norm(ns):
+            return lookup("norm", ns.kind)(ns, weights, env) if ns is not None else None
+        if spec.pre_mixer_norm is not None or spec.pre_ffn_norm is not None:
+            raise ValueError("a postnorm block has no norm in front of a sublayer")
+        self.pre_mixer = self.pre_ffn = None
+        self.post_mixer, self.post_ffn = norm(spec.post_mixer_norm), norm(spec.post_ffn_norm)
+        self.mixer = lookup("mixer", spec.mixer.kind)(spec.mixer, weights, env)
+        self.ffn = lookup("ffn", spec.ffn.kind)(spec.ffn, weights, env) if spec.ffn is not None else None
+        self.hidden = spec.mixer.hidden
+
+    @classmethod
+    def tensor_needs(cls, spec: LayerSpec) -> List[TensorNeed]:
+        needs: List[TensorNeed] = []
+        for ns in (spec.post_mixer_norm, spec.post_ffn_norm):
+            if ns is not None:
+                needs += lookup("norm", ns.kind).tensor_needs(ns)
+        needs += lookup("mixer", spec.mixer.kind).tensor_needs(spec.mixer)
+        if spec.ffn is not None:
+            needs += lookup("ffn", spec.ffn.kind).tensor_needs(spec.ffn)
+        return needs
+
+    def forward(self, h: torch.Tensor, pending: Pending, step, memory: int, writes: bool) -> Pending:
+        x = self.env.workspace.get("normed", h.shape[0], self.hidden, self.env.dtype)
+        rows_as_they_are(h, pending, x)
+        pending = (self.mixer.forward(x, step, memory, writes), self.post_mixer)
+        if self.ffn is None:
+            return pending
+        rows_as_they_are(h, pending, x)
+        return (self.ffn.forward(x, step), self.post_ffn)
+
+
 register("block", "sandwich", SandwichBlock)
+register("block", "postnorm", PostNormBlock)
 register("block", "prenorm", PreNormBlock)

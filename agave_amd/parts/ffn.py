@@ -67,7 +67,7 @@ class GatedFfn:
         act = self.env.workspace.get(tag + "_act", n, ff, x.dtype)
         if not self.gate_up.forward_geglu(x, act):
             gu = self.gate_up.forward(x, tag="gate_up" if tag == "ffn" else tag + "_gate_up")
-            kernels.gated_act(gu[:, :ff], gu[:, ff:], act, self.spec.activation)
+            kernels.gated_act(gu[:, :ff], gu[:, ff:], act, self.spec.activation, self.spec.act_limit, self.spec.act_alpha)
         return self.down.forward(act, tag=tag + "_down", slices_ok=slices_ok)    # the block adds it to the residual stream
 
 

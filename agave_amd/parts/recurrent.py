@@ -15,6 +15,12 @@ square per head, times a gain shared by the heads, times ``sigmoid(W_gate_out (W
 ``f = lower + (1 - lower) * sigmoid(W_f x + b_f)``, ``a = f``, ``k = 1 - f``, ``u = v = W_v x``; the
 read-out gets an RMS norm per head with a gain shared by the heads.
 
+``mamba2`` (a state-space mixer with one decay per head and token): one product gives ``[z | xs | B | C | dt]``;
+``xs``, ``B`` and ``C`` pass one short causal convolution with a bias and SiLU; ``d = softplus(dt + dt_bias)``;
+``a = exp(-exp(A_log_h) d)`` for every key channel, ``k = B`` and ``q = C`` of the head's group, ``u = d xs``; the
+read-out gets ``D_h xs`` on top, is multiplied by ``silu(z)``, divided by its root mean square in equal parts of the
+row, and multiplied by a weight.
+
 The gates, decays, unit vectors and the state are 32-bit whatever the engine's element type; the
 first products write 32-bit rows for that reason.
 """
@@ -25,7 +31,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..cache import GroupKey, StateNeed
-from ..config.spec import GatedDeltaSpec, Hgrn2Spec
+from ..config.spec import GatedDeltaSpec, Hgrn2Spec, Mamba2Spec
 from ..ops import sequence as seq_ops
 from ..weights.loader import TensorNeed
 from .base import BuildEnv, register, state_tensor
@@ -180,5 +186,66 @@ class Hgrn2:
         return self.o.forward(ctx, tag="hgrn2_o", slices_ok=True)
 
 
+class Mamba2:
+    @staticmethod
+    def kernel_libraries(spec, dtype):
+        return ("sequence",)
+
+    def __init__(self, spec: Mamba2Spec, weights, env: BuildEnv):
+        s = spec
+        if s.n_heads % s.groups:
+            raise ValueError("mamba2: heads must be a multiple of the groups of B and C")
+        self.inner, self.gn = s.n_heads * s.v_head_dim, s.groups * s.state
+        if self.inner % s.norm_groups:
+            raise ValueError(f"mamba2: rows of {self.inner} do not split into {s.norm_groups} equal parts for the norm")
+        self.spec, self.env = spec, env
+        self.channels = self.inner + 2 * self.gn
+        self.proj = Linear([weights.get(s.in_proj)], env, "mamba_in")
+        self.conv = ShortConv([weights.get(s.conv)], env, silu=True, name="mamba_conv",
+                              bias=weights.get(s.conv_bias) if s.conv_bias else None)
+        if self.conv.channels != self.channels:
+            raise ValueError(f"mamba2: the convolution has {self.conv.channels} channels, xs, B and C have {self.channels}")
+        self.a_log, self.dt_bias, self.skip = (_vec(weights, n, env) for n in (s.a_log, s.dt_bias, s.d_skip))
+        self.norm_weight = _vec(weights, s.out_norm, env)
+        self.o = Linear([weights.get(s.o_proj)], env, "mamba_o")
+
+    @staticmethod
+    def tensor_needs(spec: Mamba2Spec) -> List[TensorNeed]:
+        s = spec
+        inner, gn = s.n_heads * s.v_head_dim, s.groups * s.state
+        needs = [TensorNeed(s.in_proj, (2 * inner + 2 * gn + s.n_heads, s.hidden)),
+                 TensorNeed(s.conv, (inner + 2 * gn, s.conv_taps))]
+        if s.conv_bias:
+            needs.append(TensorNeed(s.conv_bias, (inner + 2 * gn,)))
+        needs += [TensorNeed(s.dt_bias, (s.n_heads,)), TensorNeed(s.a_log, (s.n_heads,)), TensorNeed(s.d_skip, (s.n_heads,)),
+                  TensorNeed(s.out_norm, (inner,)), TensorNeed(s.o_proj, (s.hidden, inner))]
+        return needs
+
+    def kv_need(self) -> Optional[GroupKey]:
+        return None
+
+    def state_need(self) -> Dict[str, StateNeed]:
+        s = self.spec
+        return {"S": StateNeed((s.n_heads, s.v_head_dim, s.state), torch.float32), "conv": self.conv.state_need()}
+
+    def forward(self, x: torch.Tensor, step, memory: int, writes: bool = True) -> torch.Tensor:
+        s, ws = self.spec, self.env.workspace
+        n = x.shape[0]
+        if not writes:
+            raise ValueError("a recurrent mixer advances its own state; it cannot read another run's")
+        proj = self.proj.forward(x, out_dtype=torch.float32, tag="mamba_in")
+        z, xbc, dt = ws.columns(proj, (0, self.inner, self.inner + self.channels, self.inner + self.channels + s.n_heads))
+        conved = ws.get("mamba_conved", n, self.channels, torch.float32)
+        self.conv.forward(xbc, conved, state_tensor(step, memory, "conv"), step)
+        xs, b, c = ws.columns(conved, (0, self.inner, self.inner + self.gn, self.channels))
+        y = ws.get("mamba_readout", n, self.inner, torch.float32)
+        seq_ops.gated_recurrence(seq_ops.SSD, c, b, xs, y, state_tensor(step, memory, "S"), step, s.n_heads, s.groups,
+                                 s.state, s.v_head_dim, dt_in=dt, a_log=self.a_log, dt_bias=self.dt_bias, skip=self.skip)
+        ctx = ws.get("mamba_ctx", n, self.inner, self.env.dtype)
+        seq_ops.gated_group_norm(y, z, self.norm_weight, ctx, s.norm_groups, s.norm_eps)
+        return self.o.forward(ctx, tag="mamba_o", slices_ok=True)
+
+
 register("mixer", "gated_delta", GatedDelta)
+register("mixer", "mamba2", Mamba2)
 register("mixer", "hgrn2", Hgrn2)

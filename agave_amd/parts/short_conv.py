@@ -1,6 +1,6 @@
 """A short causal convolution over time on every channel, with its state.
 
-``y[t, c] = act(sum_j w[c, j] * u[t - taps + 1 + j, c])``: the last column of ``w`` multiplies the
+``y[t, c] = act(b[c] + sum_j w[c, j] * u[t - taps + 1 + j, c])`` (the bias ``b`` is optional): the last column of ``w`` multiplies the
 current token's input, and inputs before the sequence's start are zeros.  The last ``taps - 1``
 inputs of every sequence are kept as state, so that a sequence fed in pieces, or token by token,
 sees what a whole pass would.  Several tensors that are convolved alike (the q, k and v of one
@@ -8,7 +8,7 @@ mixer) are stacked along the channels and run as one kernel.
 """
 from __future__ import annotations
 
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
 import torch
 
@@ -18,7 +18,8 @@ from .base import BuildEnv
 
 
 class ShortConv:
-    def __init__(self, weights: Sequence[torch.Tensor], env: BuildEnv, silu: bool, name: str = "conv"):
+    def __init__(self, weights: Sequence[torch.Tensor], env: BuildEnv, silu: bool, name: str = "conv",
+                 bias: Optional[torch.Tensor] = None):
         taps = {int(w.shape[1]) for w in weights}
         if len(taps) != 1:
             raise ValueError(f"{name}: stacked convolutions must have the same number of taps, got {sorted(taps)}")
@@ -29,10 +30,15 @@ class ShortConv:
         self.channels = self.weight.shape[0]
         self.silu = bool(silu)
         self.env = env
+        self.bias = None
+        if bias is not None:
+            if tuple(bias.shape) != (self.channels,):
+                raise ValueError(f"{name}: a bias of shape {tuple(bias.shape)} for {self.channels} channels")
+            self.bias = bias.to(torch.float32).contiguous().to(env.device)
 
     def state_need(self) -> StateNeed:
         return StateNeed((self.taps - 1, self.channels), torch.float32)
 
     def forward(self, u: torch.Tensor, out: torch.Tensor, state: torch.Tensor, step) -> None:
         """``u`` and ``out``: float32 [N, channels] (column slices are fine); ``state`` is advanced."""
-        seq_ops.short_conv(u, self.weight, out, state, step, self.silu)
+        seq_ops.short_conv(u, self.weight, out, state, step, self.silu, self.bias)
