@@ -38,9 +38,9 @@ def moe(experts, top, ff, limit, shared_ff=None, shared_limit=None):
     return out
 
 
-def latent_layer(heads, dim, rot_dim, vdim, q_rank, kv_rank, base=10000.0, scale=None, kv_from=None, mlp=None):
+def latent_layer(heads, dim, rot_dim, vdim, q_rank, kv_rank, base=10000.0, scale=None, kv_from=None, mlp=None, rot_dims=None):
     m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "q_rank": q_rank, "kv_rank": kv_rank,
-         "rot": {"base": base, "dims": rot_dim}, "scale": scale if scale is not None else (dim + rot_dim) ** -0.5}
+         "rot": {"base": base, "dims": rot_dims if rot_dims is not None else rot_dim}, "scale": scale if scale is not None else (dim + rot_dim) ** -0.5}
     if kv_from is not None:
         m["kv_from"] = kv_from
     return {"type": "latent_attention", "mixer": m, "mlp": mlp}
@@ -92,7 +92,7 @@ def tensor_shapes(cfg) -> Dict[str, tuple]:
 def random_weights(cfg, seed=0, decided_routing=False) -> Dict[str, torch.Tensor]:
     """Weights rounded to bfloat16 (so that a bfloat16 folder holds exactly these).  Matrices are drawn so that a
     row's product with a vector of unit root mean square has about unit size; ``decided_routing``: the router's bias
-    spreads the experts apart, so that rounding never changes the choice."""
+    spreads the experts apart and its matrix is small, so that rounding never changes the choice."""
     g = torch.Generator().manual_seed(seed)
     w = {}
     for name, shape in tensor_shapes(cfg).items():
@@ -112,13 +112,15 @@ def random_weights(cfg, seed=0, decided_routing=False) -> Dict[str, torch.Tensor
         elif name.endswith("router.b"):
             t = torch.randn(shape, generator=g, dtype=F) * 0.3
             if decided_routing:
-                t = torch.arange(shape[0], dtype=F)[torch.randperm(shape[0], generator=g)] * 1.5
+                t = torch.arange(shape[0], dtype=F)[torch.randperm(shape[0], generator=g)] * 0.7
         elif name.endswith("conv.b"):
             t = torch.randn(shape, generator=g, dtype=F) * 0.2
         elif name.endswith("dq.norm") or name.endswith("dkv.norm") or name.endswith("mix.norm"):
             t = 1.0 + torch.randn(shape, generator=g, dtype=F) * 0.2          # plain weights
         else:
             t = torch.randn(shape, generator=g, dtype=F) * 0.2                # weights stored around zero
+        if decided_routing and name.endswith("mlp.router"):
+            t = t * 0.02
         w[name] = t.to(torch.bfloat16).to(F)
     return w
 
