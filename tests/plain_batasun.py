@@ -182,6 +182,31 @@ def silu(x):
     return x * torch.sigmoid(x)
 
 
+def state_space_steps(xs, B, C, dt, rate, skip):
+    """xs [T, H, P], B and C [T, G, N] (head h reads group h // (H / G)), dt [T, H] (already positive), rate and skip
+    [H]:  S_t = exp(-rate dt) S_(t-1) + dt B_t xs_t^T,  y_t = S_t^T C_t + skip xs_t.  Returns (y [T, H, P], the last
+    states [H, N, P])."""
+    T, H, P_ = xs.shape
+    G, N = B.shape[1], B.shape[2]
+    y = torch.zeros(T, H, P_, dtype=F)
+    last = torch.zeros(H, N, P_, dtype=F)
+    for h in range(H):
+        g = h // (H // G)
+        S = torch.zeros(N, P_, dtype=F)
+        for t in range(T):
+            S = torch.exp(-rate[h] * dt[t, h]) * S + dt[t, h] * torch.outer(B[t, g], xs[t, h])
+            y[t, h] = S.T @ C[t, g] + skip[h] * xs[t, h]
+        last[h] = S
+    return y, last
+
+
+def gated_norm_in_parts(y, z, weight, parts, eps):
+    """y silu(z), each of the row's ``parts`` equal parts divided by its own root mean square, times ``weight``."""
+    T, width = y.shape
+    g = y * silu(z)
+    return rms(g.view(T, parts, width // parts), eps).reshape(T, width) * weight
+
+
 def mamba2(m, w, p, x, eps):
     T, H, P_, N, G = x.shape[0], m["heads"], m["vdim"], m["state"], m["groups"]
     inner, gn = H * P_, G * N
@@ -190,18 +215,8 @@ def mamba2(m, w, p, x, eps):
     xbc = silu(causal_conv(xbc, w[p + "conv"], w[p + "conv.b"]))
     xs, B, C = xbc[:, :inner].view(T, H, P_), xbc[:, inner:inner + gn].view(T, G, N), xbc[:, inner + gn:].view(T, G, N)
     dt = torch.nn.functional.softplus(dt + w[p + "dt_bias"], threshold=1e9)
-    rate = torch.exp(w[p + "A_log"])
-    y = torch.zeros(T, H, P_, dtype=F)
-    for h in range(H):
-        g = h // (H // G)
-        S = torch.zeros(N, P_, dtype=F)
-        for t in range(T):
-            S = torch.exp(-rate[h] * dt[t, h]) * S + dt[t, h] * torch.outer(B[t, g], xs[t, h])
-            y[t, h] = S.T @ C[t, g] + w[p + "D"][h] * xs[t, h]
-    y = y.reshape(T, inner) * silu(z)
-    parts = m["norm_groups"]
-    y = rms(y.view(T, parts, inner // parts), eps).reshape(T, inner) * w[p + "norm"]
-    return y @ w[p + "o"].T
+    y, _ = state_space_steps(xs, B, C, dt, torch.exp(w[p + "A_log"]), w[p + "D"])
+    return gated_norm_in_parts(y.reshape(T, inner), z, w[p + "norm"], m["norm_groups"], eps) @ w[p + "o"].T
 
 
 def expert(w, p, x, limit):

@@ -64,10 +64,17 @@ def engine(folder, dtype, **kw):
 
 
 def close(got, ref, dtype, what):
+    """32-bit: every row within 3e-5 of the largest logit.  bfloat16: rounding is what it is, and a row whose norms
+    divide by something small carries several times the usual error (the 32-bit engine's largest error sits in the
+    same rows): 4 % of the largest logit for all rows but one in twenty, twice that for those."""
     scale = float(ref.abs().max())
     err = (got.double() - ref).abs().max(dim=-1).values
-    tol = 3e-5 if dtype == "float32" else 0.04
-    assert float(err.max()) <= tol * scale, f"{what}: error {float(err.max()):.3e} of {scale:.3e} at row {int(err.argmax())}"
+    where = f"{what}: error {float(err.max()):.3e} of {scale:.3e} at row {int(err.argmax())}"
+    if dtype == "float32":
+        assert float(err.max()) <= 3e-5 * scale, where
+    else:
+        assert float(err.max()) <= 0.08 * scale, where
+        assert int((err > 0.04 * scale).sum()) <= max(1, len(err) // 20), where
 
 
 def model_for(models, name, dtype):
@@ -160,29 +167,73 @@ def test_long_decoding(models):
     close(U.run_tail(eng, toks, 500), ref, "float32", "500 tokens decoded")
 
 
-def test_an_early_token_moves_late_logits():
-    """One latent layer with a sharp softmax, and one state-space layer that forgets slowly: a change of the third
-    token moves the logits 400 tokens later through either, and the engine follows, decoding or not."""
+def far_key_model(boost=40.0):
+    """One latent layer whose head 0 is made to look for one token: the unrotated key of token ``A`` is given
+    ``boost`` more score against the unrotated query of token ``Q`` than it had, by a change of rank one in head 0's
+    key matrix.  (A layer's input is a function of the token alone in a model of one layer, so the two vectors can be
+    computed ahead.)  Other tokens' latents overlap with A's by chance and get a part of the boost; A stands out by
+    more than ten among hundreds of keys."""
+    A, Q = 0, 1
+    cfg = P.config([P.latent_layer(2, 8, 8, 12, 16, 24, base=100.0, mlp=None)], vocab=60, width=32)
+    w = P.random_weights(cfg, 3)
+    m, eps = cfg["layers"][0]["mixer"], cfg["norm"]["eps"]
+    x = P.rms(w["embed"][[A, Q]], eps) * (1.0 + w["embed.norm"])
+    c_a = P.rms((x[0] @ w["l0.mix.dkv"].T)[:m["kv_rank"]], eps) * w["l0.mix.dkv.norm"]
+    cq = P.rms(x[1] @ w["l0.mix.dq"].T, eps) * w["l0.mix.dq.norm"]
+    q0 = (cq @ w["l0.mix.uq"].T).view(m["heads"], -1)[0, :m["dim"]]
+    uk = w["l0.mix.uk"].clone().view(m["heads"], m["dim"], m["kv_rank"])
+    uk[0] += boost / (m["scale"] * float(q0 @ q0) * float(c_a @ c_a)) * torch.outer(q0, c_a)
+    w["l0.mix.uk"] = uk.reshape(-1, m["kv_rank"]).to(torch.bfloat16).to(P.F)
+    return cfg, w, A, Q
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_far_key_among_hundreds(dtype):
+    """The key that the last queries look for stands at the third position, at a page's last and first place, or far
+    inside the prompt; the queries come in the prompt, in pieces of it, and decoded one by one.  Taking the key away
+    moves the logits by much more than the engine may be off."""
     from agave_amd.engine import Engine
-    for which in ("latent", "state"):
-        if which == "latent":
-            cfg = P.config([P.latent_layer(2, 8, 8, 12, 16, 24, base=100.0, scale=3.0, mlp=None)], vocab=60, width=32)
-        else:
-            cfg = P.config([P.mamba_layer(2, 8, 16, 1, 3, 2, mlp=None)], vocab=60, width=32)
-        w = P.random_weights(cfg, 3)
-        if which == "state":
-            w["l0.mix.A_log"] = torch.full((2,), -7.0, dtype=P.F)             # almost nothing is forgotten
-        eng = Engine.from_tensors(cfg, {k: v.bfloat16() for k, v in w.items()}, dtype="float32", max_slots=2, max_context=512)
-        toks = U.random_tokens(430, 60, 3)
-        other = list(toks)
-        other[2] = (toks[2] + 11) % 60
-        ref, ref_other = P.forward(cfg, w, toks), P.forward(cfg, w, other)
-        moved = float((ref[-1] - ref_other[-1]).abs().max())
-        assert moved > 1e-3 * float(ref.abs().max()), which
-        for t, r in ((toks, ref), (other, ref_other)):
-            got = U.run_tail(eng, t, 40)
-            assert float((got[-1].double() - r[-1]).abs().max()) < 0.02 * moved, which
-            close(got, r, "float32", which)
+    cfg, w, A, Q = far_key_model()
+    eng = Engine.from_tensors(cfg, {k: v.bfloat16() for k, v in w.items()}, dtype=dtype, max_slots=2, max_context=512)
+    for at in (2, 63, 64, 300):
+        toks = [2 + t % 58 for t in U.random_tokens(430, 1000, at)]
+        for t in range(380, 430, 3):
+            toks[t] = Q
+        toks[-1] = Q
+        toks[at] = A
+        without = list(toks)
+        without[at] = 7
+        ref, ref_without = P.forward(cfg, w, toks), P.forward(cfg, w, without)
+        scale = float(ref.abs().max())
+        moved = float((ref[-1] - ref_without[-1]).abs().max())
+        assert moved > 0.1 * scale, at
+        eng.prefill_chunk = 0
+        runs = {"whole": U.run_whole(eng, toks), "decoded": U.run_tail(eng, toks, 60)}
+        eng.prefill_chunk = 50
+        runs["pieces"] = U.run_whole(eng, toks)
+        for what, got in runs.items():
+            close(got, ref, dtype, f"key at {at}, {what}")
+            assert float((got[-1].double() - ref[-1]).abs().max()) < (0.002 if dtype == "float32" else 0.2) * moved, (at, what)
+
+
+def test_an_early_token_stays_in_the_state():
+    """A state-space layer that forgets slowly: a change of the third token moves the logits 400 tokens later, and the
+    engine follows, decoding or not."""
+    from agave_amd.engine import Engine
+    cfg = P.config([P.mamba_layer(2, 8, 16, 1, 3, 2, mlp=None)], vocab=60, width=32)
+    w = P.random_weights(cfg, 3)
+    w["l0.mix.A_log"] = torch.full((2,), -7.0, dtype=P.F)             # almost nothing is forgotten
+    eng = Engine.from_tensors(cfg, {k: v.bfloat16() for k, v in w.items()}, dtype="float32", max_slots=2, max_context=512)
+    toks = U.random_tokens(430, 60, 3)
+    other = list(toks)
+    other[2] = (toks[2] + 11) % 60
+    ref, ref_other = P.forward(cfg, w, toks), P.forward(cfg, w, other)
+    moved = float((ref[-1] - ref_other[-1]).abs().max())
+    assert moved > 1e-3 * float(ref.abs().max())
+    for t, r in ((toks, ref), (other, ref_other)):
+        got = U.run_tail(eng, t, 40)
+        assert float((got[-1].double() - r[-1]).abs().max()) < 0.02 * moved
+        close(got, r, "float32", "state")
 
 
 @pytest.mark.parametrize("dtype", ["float32"])
