@@ -79,13 +79,13 @@ class KVCache:
             if k.layout == "tiles" and k.v_head_dim not in (None, k.head_dim):
                 raise CacheError("pages in tile order hold keys and values of one size; a mixer with narrower "
                                  "values asks for the layout 'rows'")
-        # ("rows_vt" in bfloat16 with a key size that is a multiple of 8 and a value size that is a multiple of 16:
-        # the same, in the order the biased attention's matrix-core kernel reads its operands)
+        # ("rows_vt" in bfloat16 with a key size that is a multiple of 8, up to 576, and a value size that is a multiple
+        # of 16, up to 512: the same, in the order the biased attention's matrix-core kernel reads its operands)
         self.packed: List[bool] = [
-            dtype == torch.bfloat16 and k.head_dim <= 256 and
-            ((k.layout == "tiles" and k.head_dim % 16 == 0) or
+            dtype == torch.bfloat16 and
+            ((k.layout == "tiles" and k.head_dim % 16 == 0 and k.head_dim <= 256) or
              (k.layout == "rows_vt" and k.head_dim % 8 == 0 and (k.v_head_dim or k.head_dim) % 16 == 0
-              and (k.v_head_dim or k.head_dim) <= 256))
+              and k.head_dim <= 576 and (k.v_head_dim or k.head_dim) <= 512))
             for k in self.group_keys]
         for key, mems, packed in zip(self.group_keys, members, self.packed):
             n = pages_per_group[key]

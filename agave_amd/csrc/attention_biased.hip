@@ -119,11 +119,11 @@ __device__ __forceinline__ float score_bias(const BiasedArgs& A, int h, int dist
 
 // ------------------------------------------------------------------ plain kernel
 #define BCHUNK 256           // keys per pass = 4 pages
-#define BACC 2               // value size <= 512
+#define BACC 4               // value size <= 1024
 
 template <typename T>
 __global__ __launch_bounds__(256) void attn_biased_plain_kernel(BiasedArgs A) {
-    __shared__ float qs[512];
+    __shared__ float qs[1024];
     __shared__ float sc[BCHUNK];
     __shared__ long page_of[BCHUNK / AGAVE_PAGE];
     __shared__ float red[16];
@@ -150,7 +150,9 @@ __global__ __launch_bounds__(256) void attn_biased_plain_kernel(BiasedArgs A) {
         m = A.sink[h];
         l = 1.f;
     }
-    float acc[BACC] = {0.f, 0.f};
+    float acc[BACC];
+#pragma unroll
+    for (int a = 0; a < BACC; ++a) acc[a] = 0.f;
 
     // two stretches of keys: the kept first positions that the window has left behind, then the window
     for (int part = 0; part < 2; ++part) {
@@ -230,7 +232,7 @@ static int check_biased(const BiasedArgs& A, int N) {
     AGAVE_CHECK(N >= 0 && A.nh > 0 && A.nkv > 0 && A.hd > 0 && A.vd > 0, "attn_biased: bad sizes N=%d nh=%d nkv=%d hd=%d vd=%d", N,
                 A.nh, A.nkv, A.hd, A.vd);
     AGAVE_CHECK(A.nh % A.nkv == 0, "attn_biased: %d query heads are not a multiple of %d kv heads", A.nh, A.nkv);
-    AGAVE_CHECK(A.hd <= 512 && A.vd <= 256 * BACC, "attn_biased: head sizes %d / %d exceed 512", A.hd, A.vd);
+    AGAVE_CHECK(A.hd <= 1024 && A.vd <= 256 * BACC, "attn_biased: head sizes %d / %d exceed 1024", A.hd, A.vd);
     AGAVE_CHECK(A.ldq >= (long)A.nh * A.hd && A.ldo >= (long)A.nh * A.vd && (!A.gate || A.ldg >= (long)A.nh * A.vd),
                 "attn_biased: a row stride is too small");
     AGAVE_CHECK(A.window >= 0 && A.keep_first >= 0 && A.head >= 0, "attn_biased: negative window, kept positions or kept pages");
@@ -287,12 +289,17 @@ struct MfmaMode {
     int one_row;                 // 1: a step of one row a sequence
     const int* cu;               // [sequences + 1] first row of every sequence (many rows)
     int table_in_lds;            // the bias table's row of this head is copied to LDS (many rows)
+    int splits;                  // one row: this many workgroups share a row's pages and leave partial results
+    float* parts;                // [rows][heads][splits][2 + vd]: reference, sum, unnormalised row (splits > 1)
+    int q_off;                   // floats of LDS in front of the place for Q (the longest heads keep Q there)
 };
 
 typedef __attribute__((address_space(3))) u32x4_t lds_u32x4;
 
+// (Heads of more than 256 key or value elements hold most of a wave's registers in Q and O^T: their workgroups have
+// four waves, one a SIMD, and a wave may use the whole register file.)
 template <int KS, int VB, int NC, bool LDSP>
-__global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, MfmaMode M) {
+__global__ __launch_bounds__((KS > 8 || VB > 16) ? 256 : 512) void attn_biased_mfma_kernel(BiasedArgs A, MfmaMode M) {
     extern __shared__ float lds_generic[];
     // (every LDS access goes through a pointer that says so: no pointer may end up chosen between the two memories)
     typedef __attribute__((address_space(3))) float lds_float;
@@ -309,8 +316,9 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
     int pmin, pmax;                                 // the wave's range of positions (the same in every lane)
     int wg_first = 0, wg_last = 0;                  // the workgroup's (many rows)
     bool wave_on = true;
+    const int splits = M.one_row ? M.splits : 1, sp = M.one_row ? (int)(blockIdx.x % splits) : 0;
     if (M.one_row) {
-        row[0] = blockIdx.x;
+        row[0] = blockIdx.x / splits;
         b = A.tok_seq[row[0]];
         const int hg = blockIdx.z * 16 + c;
         valid[0] = hg < per;
@@ -364,7 +372,13 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
     if (A.bias_mode == 2) bias_row = A.bias + (size_t)head * A.bias_len;
 
     // Q as the B operand: lane holds Q[column c][32 ks + 8 g .. + 8]
-    frag16 qf[NC][KS];
+    // The longest heads (more than 12 steps) keep Q in LDS instead, in the same order, and read an operand when it is
+    // multiplied: with O^T of 512 value columns in registers there is no room for both.  A wave reads what it wrote
+    // itself (in a step of one row all waves hold the same Q and write the same place).
+    constexpr bool QL = KS > 12;
+    static_assert(!QL || NC == 1, "Q in LDS is for one block of columns a wave");
+    lds_u32x4* qs = (lds_u32x4*)(lds + M.q_off) + (M.one_row ? 0 : (size_t)w * KS * 64);
+    frag16 qf[NC][QL ? 1 : KS];
 #pragma unroll
     for (int cb = 0; cb < NC; ++cb) {
         const bf16* qrow = (const bf16*)A.q + (size_t)row[cb] * A.ldq + (size_t)head * hd;
@@ -374,7 +388,10 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
             // where it lies past the head's end: a load under a per-lane condition is waited for on the spot)
             const int k0 = 32 * ks + 8 * g;
             const uint4 got = *reinterpret_cast<const uint4*>(qrow + (k0 < hd ? k0 : 0));
-            qf[cb][ks].u = (valid[cb] && k0 < hd) ? got : make_uint4(0, 0, 0, 0);
+            frag16 f;
+            f.u = (valid[cb] && k0 < hd) ? got : make_uint4(0, 0, 0, 0);
+            if constexpr (QL) qs[ks * 64 + lane] = f.r;
+            else qf[cb][ks] = f;
         }
     }
 
@@ -386,13 +403,13 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
         for (int nb = 0; nb < VB; ++nb) o[cb][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         m[cb] = -INFINITY;
         l[cb] = 0.f;
-        if (A.sink && (!M.one_row || w == 0)) {
+        if (A.sink && (!M.one_row || (w == 0 && sp == 0))) {
             m[cb] = A.sink[head] * LOG2E;
             l[cb] = g == 0 ? 1.f : 0.f;         // the lane groups' sums are added up at the end
         }
     }
 
-    const int stride = M.one_row ? nw : 1;
+    const int stride = M.one_row ? nw * splits : 1;
     auto page_of = [&](int idx) -> long {
         if (idx >= n_pg) return -1;
         const int pi = idx < n_kept ? idx : first_win + idx - n_kept;
@@ -433,17 +450,32 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
             // (a whole operand in one load of a kilobyte; steps past the head's end read step 0 again and are emptied)
-            frag16 kf[KS];
+            // (a long head's steps come in two or three batches, so that no more than six or nine operands wait in registers; the
+            // compiler is told not to move anything across the batches' border, or it asks for all of them at once)
+            constexpr int KCH = KS > 12 ? 6 : KS > 9 ? (KS + 1) / 2 : KS;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const u32x4_t got = kt[(kb * ksl + (ks < ksl ? ks : 0)) * 64 + lane];
-                kf[ks].r = ks < ksl ? got : u32x4_t{0u, 0u, 0u, 0u};
-            }
+            for (int cb = 0; cb < NC; ++cb) s[cb][kb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int cb = 0; cb < NC; ++cb) {
-                s[cb][kb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            for (int k0 = 0; k0 < KS; k0 += KCH) {
+                frag16 kf[KCH];
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) s[cb][kb] = mfma_16x16x32(kf[ks], qf[cb][ks], s[cb][kb]);
+                for (int kk = 0; kk < KCH; ++kk) {
+                    const int ks = k0 + kk;
+                    const u32x4_t got = kt[(kb * ksl + (ks < ksl ? ks : 0)) * 64 + lane];
+                    kf[kk].r = ks < ksl ? got : u32x4_t{0u, 0u, 0u, 0u};
+                }
+#pragma unroll
+                for (int cb = 0; cb < NC; ++cb) {
+#pragma unroll
+                    for (int kk = 0; kk < KCH; ++kk)
+                        if (k0 + kk < KS) {
+                            frag16 qv;
+                            if constexpr (QL) qv.r = qs[(k0 + kk) * 64 + lane];
+                            else qv = qf[cb][k0 + kk];
+                            s[cb][kb] = mfma_16x16x32(kf[kk], qv, s[cb][kb]);
+                        }
+                }
+                if constexpr (KS > 9) __builtin_amdgcn_sched_barrier(0);
             }
         }
         // Scale, bias, mask and softmax, a column block at a time, in the base-2 domain (scale, slopes, table and
@@ -532,6 +564,9 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
                     o[cb][nb] = mfma_16x16x32(vf[1], pf[cb][1], o[cb][nb]);
                 }
             }
+            if constexpr (VB > 16) {                    // (four blocks' value operands at a time, see above)
+                if ((nb & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+            }
         }
     };
 
@@ -583,7 +618,7 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
         }
         if (!wave_on) return;
     } else {
-        int idx = M.one_row ? w : 0;
+        int idx = M.one_row ? sp * nw + w : 0;
         long pg = page_of(idx);
         for (; idx < n_pg; idx += stride) {
             const long pg_next = page_of(idx + stride);         // asked for now, used in the next turn
@@ -632,6 +667,24 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
 #pragma unroll
                 for (int e = 0; e < 4; ++e) o[0][nb][e] = o[0][nb][e] * a1 + other[32 + (16 * nb + 4 * g + (e ^ (g & 1))) * 16 + c] * a2;
         }
+        if (splits > 1) {
+            // this workgroup's share of the row: reference, sum and the unnormalised sums over the values
+            if (!valid[0]) return;
+            float* mine = M.parts + (((size_t)row[0] * nh + head) * splits + sp) * (size_t)(vd + 2);
+            if (g == 0) {
+                mine[0] = m[0];
+                mine[1] = l[0];
+            }
+#pragma unroll
+            for (int nb = 0; nb < VB; ++nb) {
+                const int d0 = 16 * nb + 4 * g;
+                if (d0 < vd) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) mine[2 + d0 + e] = o[0][nb][e];
+                }
+            }
+            return;
+        }
     }
 #pragma unroll
     for (int cb = 0; cb < NC; ++cb) {
@@ -658,6 +711,32 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
     }
 }
 
+// The shares of a row that several workgroups left: a workgroup per (row, head), a thread per value column.
+__global__ __launch_bounds__(256) void attn_biased_merge_kernel(const float* __restrict__ parts, int splits, int nh, int vd,
+                                                                bf16* __restrict__ out, long ldo, const bf16* __restrict__ gate,
+                                                                long ldg) {
+    const int t = blockIdx.x / nh, h = blockIdx.x % nh;
+    const float* mine = parts + (size_t)blockIdx.x * splits * (vd + 2);
+    float mx = -INFINITY;
+    for (int s = 0; s < splits; ++s) mx = fmaxf(mx, mine[(size_t)s * (vd + 2)]);
+    float total = 0.f;
+    for (int s = 0; s < splits; ++s) {
+        const float ms = mine[(size_t)s * (vd + 2)];
+        if (ms != -INFINITY) total += mine[(size_t)s * (vd + 2) + 1] * __builtin_amdgcn_exp2f(ms - mx);
+    }
+    const float inv = total > 0.f ? 1.0f / total : 0.f;
+    for (int d = threadIdx.x; d < vd; d += blockDim.x) {
+        float acc = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            const float ms = mine[(size_t)s * (vd + 2)];
+            if (ms != -INFINITY) acc = fmaf(mine[(size_t)s * (vd + 2) + 2 + d], __builtin_amdgcn_exp2f(ms - mx), acc);
+        }
+        float y = acc * inv;
+        if (gate) y *= 1.0f / (1.0f + __expf(-bf16_to_f32(gate[(size_t)t * ldg + (size_t)h * vd + d])));
+        out[(size_t)t * ldo + (size_t)h * vd + d] = f32_to_bf16(y);
+    }
+}
+
 template <int KS, int VB>
 static int launch_biased_mfma(const BiasedArgs& A, const MfmaMode& M, dim3 grid, int threads, int nc, size_t lds_bytes,
                               hipStream_t stream) {
@@ -673,6 +752,15 @@ static int launch_biased_mfma(const BiasedArgs& A, const MfmaMode& M, dim3 grid,
             attn_biased_mfma_kernel<KS, VB, 2, true><<<grid, threads, lds_bytes, stream>>>(A, M);
         }
     } else {
+        if (lds_bytes > 64 * 1024) {
+            static bool raised1 = false;            // (the waves' partial results of a wide value head)
+            if (!raised1) {
+                AGAVE_CHECK(hipFuncSetAttribute((const void*)attn_biased_mfma_kernel<KS, VB, 1, false>,
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024) == hipSuccess,
+                            "attn_biased_mfma: cannot raise the LDS allowance");
+                raised1 = true;
+            }
+        }
         attn_biased_mfma_kernel<KS, VB, 1, false><<<grid, threads, lds_bytes, stream>>>(A, M);
     }
     return 0;
@@ -688,7 +776,7 @@ static int launch_biased_mfma(const BiasedArgs& A, const MfmaMode& M, dim3 grid,
 
 // 1 if the matrix-core kernel takes these sizes (the caller then may call it), else 0
 extern "C" int agave_attn_biased_mfma_ok(int hd, int vd, int ldq, int ldo, int ldg) {
-    return (hd % 8 == 0 && hd <= 256 && vd % 16 == 0 && vd <= 256 && ldq % 8 == 0 && ldo % 4 == 0 && ldg % 4 == 0) ? 1 : 0;
+    return (hd % 8 == 0 && hd <= 576 && vd % 16 == 0 && vd <= 512 && ldq % 8 == 0 && ldo % 4 == 0 && ldg % 4 == 0) ? 1 : 0;
 }
 
 // `cu`: first row of every sequence (device, sequences + 1 entries), used by steps of many rows;
@@ -698,19 +786,23 @@ extern "C" int agave_attn_biased_mfma(const void* q, long ldq, void* out, long l
                                       int head, int n_pages, const int* tok_seq, const int* tok_pos, const int* cu, int N,
                                       int n_seqs, int max_rows, int one_row, int nh, int nkv, int hd, int vd, float scale,
                                       int window, int keep_first, int bias_mode, const float* bias, int bias_len,
-                                      const float* sink, hipStream_t stream) {
+                                      const float* sink, int splits, float* parts, hipStream_t stream) {
     BiasedArgs A{q, ldq, out, ldo, gate, ldg, k_pages, v_pages, table, width, base, head, n_pages, tok_seq, tok_pos,
                  nh, nkv, hd, vd, scale, window, keep_first, bias_mode, bias, bias_len, sink, 1};
     if (check_biased(A, N)) return -1;
+    AGAVE_CHECK(splits >= 1 && splits <= 64 && (splits == 1 || (one_row && parts)),
+                "attn_biased_mfma: %d shares of a row (1 to 64, in steps of one row a sequence, with memory for them)", splits);
     AGAVE_CHECK(agave_attn_biased_mfma_ok(hd, vd, (int)(ldq % 8), (int)(ldo % 4), (int)(ldg % 4)),
                 "attn_biased_mfma: head sizes %d / %d or row strides that the matrix-core kernel does not take", hd, vd);
     AGAVE_CHECK(((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0 && ((uintptr_t)gate % 8) == 0 && (nh * (long)hd) % 8 == 0,
                 "attn_biased_mfma: rows must be aligned to 16 bytes");
     AGAVE_CHECK(cu && n_seqs > 0 && max_rows > 0 && (!one_row || N == n_seqs), "attn_biased_mfma: bad step");
     if (N == 0) return 0;
-    const int ks = hd <= 32 ? 1 : hd <= 64 ? 2 : hd <= 128 ? 4 : 8;
-    const int vb = vd <= 32 ? 2 : vd <= 64 ? 4 : vd <= 128 ? 8 : 16;
-    MfmaMode M{one_row, cu, 0};
+    // (heads beyond 256 come in two sizes of both at once: up to 384 / 384 and up to 576 / 512)
+    const bool wide = hd > 256 || vd > 256, widest = hd > 384 || vd > 384;
+    const int ks = wide ? (widest ? 18 : 12) : hd <= 32 ? 1 : hd <= 64 ? 2 : hd <= 128 ? 4 : 8;
+    const int vb = wide ? (widest ? 32 : 24) : vd <= 32 ? 2 : vd <= 64 ? 4 : vd <= 128 ? 8 : 16;
+    MfmaMode M{one_row, cu, 0, splits, parts, 0};
     dim3 grid;
     size_t lds_bytes = 0;
     int threads = 256, nc = 1;
@@ -719,7 +811,7 @@ extern "C" int agave_attn_biased_mfma(const void* q, long ldq, void* out, long l
         const int per = nh / nkv;
         const int nw = vb <= 8 ? 8 : 4;
         threads = 64 * nw;
-        grid = dim3(N, nkv, (per + 15) / 16);
+        grid = dim3(N * splits, nkv, (per + 15) / 16);
         lds_bytes = (size_t)(nw - 1) * (vb * 16 * 16 + 32) * sizeof(float);
     } else {
         // 32 rows a wave where the step is long enough to fill the chip that way and the registers allow
@@ -739,14 +831,25 @@ extern "C" int agave_attn_biased_mfma(const void* q, long ldq, void* out, long l
         grid = dim3((max_rows + 64 * nc - 1) / (64 * nc), n_seqs, nh);
         AGAVE_CHECK(grid.y <= 65535 && grid.z <= 65535, "attn_biased_mfma: too many sequences or heads for the grid");
     }
+    if (ks > 12) {                                      // Q in LDS, behind whatever else is there
+        M.q_off = (int)(lds_bytes / sizeof(float));
+        lds_bytes += (size_t)(one_row ? 1 : threads / 64) * ks * 1024;
+    }
     int rc = 0;
     switch (ks) {
         case 1: BIASED_VB(1); break;
         case 2: BIASED_VB(2); break;
         case 4: BIASED_VB(4); break;
-        default: BIASED_VB(8); break;
+        case 8: BIASED_VB(8); break;
+        case 12: rc = launch_biased_mfma<12, 24>(A, M, grid, threads, nc, lds_bytes, stream); break;
+        default: rc = launch_biased_mfma<18, 32>(A, M, grid, threads, nc, lds_bytes, stream); break;
     }
     if (rc) return rc;
     AGAVE_LAUNCH_CHECK("attn_biased_mfma");
+    if (splits > 1) {
+        attn_biased_merge_kernel<<<N * nh, vd <= 64 ? 64 : vd <= 128 ? 128 : 256, 0, stream>>>(parts, splits, nh, vd, (bf16*)out, ldo,
+                                                                                      (const bf16*)gate, ldg);
+        AGAVE_LAUNCH_CHECK("attn_biased_merge");
+    }
     return 0;
 }

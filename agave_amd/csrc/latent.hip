@@ -138,7 +138,7 @@ __global__ __launch_bounds__(256) void heads_product_plain_kernel(HeadsProductAr
 }
 
 // The matrix cores' form (bfloat16; K a multiple of 8, aligned rows): a workgroup takes 64 tokens of one head and 64
-// output columns; each of its four waves 16 tokens against the 64 columns, both operands straight from memory in the
+// output columns (or, in a step of up to 16 tokens, those tokens and 256 columns); each of its four waves 16 tokens against 64 columns, both operands straight from memory in the
 // order v_mfma_f32_16x16x32_bf16 reads them (a lane's eight neighbours along K are 16 bytes of a row).  The head's
 // weights are small and stay in the caches; what the kernel moves is the rows.  The trailing elements are copied,
 // rotated, by the workgroups of the first column block.
@@ -146,8 +146,12 @@ __global__ __launch_bounds__(256) void heads_product_mfma_kernel(HeadsProductArg
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int h = blockIdx.y;
-    const int row0 = blockIdx.x * 64 + wv * 16, col0 = blockIdx.z * 64;
+    // up to 16 tokens (a decode step): the four waves take four blocks of columns of the same 16 rows
+    const bool few = A.n_tokens <= 16;
+    const int row0 = few ? 0 : blockIdx.x * 64 + wv * 16;
+    const int col0 = few ? (blockIdx.z * 4 + wv) * 64 : blockIdx.z * 64;
     const int K = A.K, n_out = A.n_out;
+    if (col0 >= n_out || row0 >= A.n_tokens) return;            // (no barrier below)
     const bf16* x = (const bf16*)A.x;
     const bf16* w = (const bf16*)A.w + (size_t)h * n_out * K;
     bf16* y = (bf16*)A.y;
@@ -190,7 +194,7 @@ __global__ __launch_bounds__(256) void heads_product_mfma_kernel(HeadsProductArg
             y[(size_t)t * A.ldy + (size_t)h * A.ys + col] = f32_to_bf16(v);
         }
     }
-    if (A.tail && blockIdx.z == 0) {
+    if (A.tail && col0 == 0) {
         for (int i = lane; i < 16 * A.tail; i += 64) {
             const int t = row0 + i / A.tail, e = i % A.tail;
             if (t >= A.n_tokens) continue;
@@ -222,9 +226,9 @@ extern "C" int agave_heads_product(int dtype, const void* x, long ldx, int xs, c
     if (n_tokens == 0) return 0;
     HeadsProductArgs A{x, ldx, xs, w, y, ldy, ys, gate, ldg, freq, rot_half, tail, tok_pos, n_tokens, heads, n_out, K};
     const bool mfma = !plain && dtype == AGAVE_BF16 && K % 8 == 0 && xs % 8 == 0 && ldx % 8 == 0 &&
-                      ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0 && n_tokens >= 16;
+                      ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
     if (mfma) {
-        const dim3 grid((n_tokens + 63) / 64, heads, (n_out + 63) / 64);
+        const dim3 grid = n_tokens <= 16 ? dim3(1, heads, (n_out + 255) / 256) : dim3((n_tokens + 63) / 64, heads, (n_out + 63) / 64);
         AGAVE_CHECK(grid.z <= 65535, "heads_product: too many columns");
         heads_product_mfma_kernel<<<grid, 256, 0, stream>>>(A);
     } else {

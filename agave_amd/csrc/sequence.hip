@@ -1020,24 +1020,47 @@ extern "C" int agave_head_norm_gate(int dtype, const float* o, long ldo_in, cons
 }
 
 // ------------------------------------------------------------------ a gate, then a norm in equal parts of the row
-//   g = y * silu(z);  out = g / sqrt(mean over the part (g^2) + eps) * w     (a wave per (token, part); w is [parts * size])
+//   g = y * silu(z);  out = g / sqrt(mean over the part (g^2) + eps) * w     (w is [parts * size])
+// A workgroup per (token, part), of one to four waves by the part's size; a thread keeps up to eight gated values in
+// registers between the sum of squares and the output (longer parts are computed twice).
 template <typename T>
-__global__ __launch_bounds__(64) void gated_group_norm_kernel(const float* __restrict__ y, long ldy, const float* __restrict__ z,
-                                                              long ldz, const float* __restrict__ w, T* __restrict__ out, long ldo,
-                                                              int parts, int size, float eps) {
-    const int t = blockIdx.x / parts, g = blockIdx.x % parts, lane = threadIdx.x;
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ y, long ldy, const float* __restrict__ z,
+                                                               long ldz, const float* __restrict__ w, T* __restrict__ out, long ldo,
+                                                               int parts, int size, float eps) {
+    __shared__ float red[8];
+    constexpr int KEEP = 8;
+    const int t = blockIdx.x / parts, g = blockIdx.x % parts, tid = threadIdx.x, nt = blockDim.x;
     const float* yr = y + (size_t)t * ldy + (size_t)g * size;
     const float* zr = z + (size_t)t * ldz + (size_t)g * size;
+    const float* wr = w + (size_t)g * size;
+    float yv[KEEP], zv[KEEP], gv[KEEP];
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {                    // (loads from inside the part, emptied afterwards)
+        const int e = tid + i * nt;
+        yv[i] = yr[e < size ? e : 0];
+        zv[i] = zr[e < size ? e : 0];
+    }
     float ss = 0.f;
-    for (int e = lane; e < size; e += 64) {
-        const float zv = zr[e], v = yr[e] * (zv / (1.0f + expf(-zv)));
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {
+        gv[i] = tid + i * nt < size ? yv[i] * (zv[i] / (1.0f + expf(-zv[i]))) : 0.f;
+        ss = fmaf(gv[i], gv[i], ss);
+    }
+    for (int e = tid + KEEP * nt; e < size; e += nt) {
+        const float zz = zr[e], v = yr[e] * (zz / (1.0f + expf(-zz)));
         ss = fmaf(v, v, ss);
     }
-    ss = wave_sum(ss);
+    ss = nt > 64 ? block_sum(ss, red) : wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)size + eps);
-    for (int e = lane; e < size; e += 64) {
-        const float zv = zr[e], v = yr[e] * (zv / (1.0f + expf(-zv)));
-        st(out + (size_t)t * ldo + (size_t)g * size + e, v * inv * w[(size_t)g * size + e]);
+    T* o = out + (size_t)t * ldo + (size_t)g * size;
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {
+        const int e = tid + i * nt;
+        if (e < size) st(o + e, gv[i] * inv * wr[e]);
+    }
+    for (int e = tid + KEEP * nt; e < size; e += nt) {
+        const float zz = zr[e], v = yr[e] * (zz / (1.0f + expf(-zz)));
+        st(o + e, v * inv * wr[e]);
     }
 }
 
@@ -1048,10 +1071,11 @@ extern "C" int agave_gated_group_norm(int dtype, const float* y, long ldy, const
     AGAVE_CHECK(y && z && w && out && ldy >= width && ldz >= width && ldo >= width, "gated_group_norm: bad buffers");
     AGAVE_CHECK((long)N * parts < 2147483647L, "gated_group_norm: too many rows");
     if (N == 0) return 0;
+    const int threads = size <= 256 ? 64 : size <= 1024 ? 128 : 256;
     if (dtype == AGAVE_F32)
-        gated_group_norm_kernel<float><<<N * parts, 64, 0, stream>>>(y, ldy, z, ldz, w, (float*)out, ldo, parts, size, eps);
+        gated_group_norm_kernel<float><<<N * parts, threads, 0, stream>>>(y, ldy, z, ldz, w, (float*)out, ldo, parts, size, eps);
     else if (dtype == AGAVE_BF16)
-        gated_group_norm_kernel<bf16><<<N * parts, 64, 0, stream>>>(y, ldy, z, ldz, w, (bf16*)out, ldo, parts, size, eps);
+        gated_group_norm_kernel<bf16><<<N * parts, threads, 0, stream>>>(y, ldy, z, ldz, w, (bf16*)out, ldo, parts, size, eps);
     else
         AGAVE_CHECK(false, "gated_group_norm: unknown dtype %d", dtype);
     AGAVE_LAUNCH_CHECK("gated_group_norm");

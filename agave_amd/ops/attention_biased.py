@@ -16,6 +16,17 @@ from .kernels import _P, _I, _L, _F, _dev, _f32vec, _i32, _rows, dt, ptr, stream
 LIBRARY = "attention_biased"
 
 BIAS_NONE, BIAS_SLOPES, BIAS_TABLE = 0, 1, 2
+MFMA_MAX_KEY, MFMA_MAX_VALUE = 576, 512         # the largest heads the matrix-core kernel takes
+MAX_SPLITS = 16
+
+
+def decode_splits(n_rows: int, n_kv: int, per: int, v_head_dim: int, table_width: int) -> int:
+    """How many workgroups share the pages of one (row, key head) in a step of one row a sequence: enough to have some
+    two hundred workgroups at work, never more than the longest sequence's pages give every wave one.  It depends on
+    nothing that changes from step to step, so a recorded step stays valid."""
+    waves = 8 if v_head_dim <= 128 else 4
+    groups = max(1, n_rows * n_kv * ((per + 15) // 16))
+    return max(1, min(MAX_SPLITS, 192 // groups, -(-table_width // waves)))
 
 kernels.register_signatures(LIBRARY, {
     "agave_kv_append_rows": [_I, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P],
@@ -23,7 +34,7 @@ kernels.register_signatures(LIBRARY, {
                                 _I, _I, _I, _P, _I, _P, _I, _P],
     "agave_attn_biased_mfma_ok": [_I, _I, _I, _I, _I],
     "agave_attn_biased_mfma": [_P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I,
-                               _F, _I, _I, _I, _P, _I, _P, _P],
+                               _F, _I, _I, _I, _P, _I, _P, _I, _P, _P],
 })
 
 
@@ -33,8 +44,9 @@ def _lib():
 
 def _check_row_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, nkv: int, hd: int, vd: int, dtype: torch.dtype,
                      packed: bool = False) -> int:
-    if packed and (dtype != torch.bfloat16 or hd % 8 or vd % 16 or hd > 256 or vd > 256):
-        raise ValueError("pages in operand order hold bfloat16, keys in steps of 8 and values in steps of 16, up to 256")
+    if packed and (dtype != torch.bfloat16 or hd % 8 or vd % 16 or hd > MFMA_MAX_KEY or vd > MFMA_MAX_VALUE):
+        raise ValueError(f"pages in operand order hold bfloat16, keys in steps of 8 up to {MFMA_MAX_KEY} and values in steps "
+                         f"of 16 up to {MFMA_MAX_VALUE}")
     hd_k = (hd + 31) // 32 * 32 if packed else hd       # operands are whole steps of 32 along the head
     if k_pages.dim() != 4 or tuple(k_pages.shape[1:]) != (nkv, 64, hd_k) or not k_pages.is_contiguous():
         raise ValueError(f"K pages must be contiguous [pages, {nkv}, 64, {hd_k}], got {tuple(k_pages.shape)}")
@@ -72,14 +84,16 @@ def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], 
               v_pages: torch.Tensor, table: torch.Tensor, base: torch.Tensor, head: int, step, n_heads: int, n_kv: int,
               head_dim: int, v_head_dim: int, scale: float, window: Optional[int], keep_first: int, bias_mode: int,
               bias: Optional[torch.Tensor], sink: Optional[torch.Tensor], packed: bool = False,
-              force_plain: bool = False) -> None:
+              force_plain: bool = False, workspace=None, splits: Optional[int] = None) -> None:
     """out[t, h] = sum_j w_j v_j with w = softmax_j(scale q.k_j + bias(h, p - j)) over the keys that token t at
     position p sees (j <= p and (p - j < window or j < keep_first)), the sink's exp(sink_h) added to the
     denominator, times sigmoid(gate[t, h]) element by element.  ``bias``: slopes [heads] (``BIAS_SLOPES``:
     the bias is -slope_h (p - j)) or a table [heads, distances] (``BIAS_TABLE``: distances beyond the table take
     its last column).  Pages in operand order (``packed``: bfloat16, a key size that is a multiple of 8 and a value size
-    that is a multiple of 16, both up to 256) run on the matrix cores, everything else (and everything with
-    ``force_plain``) on the plain kernel, which reads either order."""
+    that is a multiple of 16, up to 576 and 512) run on the matrix cores, everything else (and everything with
+    ``force_plain``) on the plain kernel, which reads either order.  With a ``workspace`` (something with
+    ``get(name, rows, cols, dtype)``) a step of one row a sequence may share a row's pages among several workgroups,
+    whose partial results a second kernel merges (``splits``: how many; None: :func:`decode_splits`)."""
     _dev(q, out, gate, k_pages, v_pages, table, base, bias, sink)
     n = step.n_tokens
     ldq, ldo = _rows(q, "q"), _rows(out, "out")
@@ -109,10 +123,20 @@ def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], 
         _i32(step.cu_dev, "cu", step.n_seqs + 1)
         max_rows = max(b - a for a, b in zip(step.cu[:-1], step.cu[1:]))
         one_row = 1 if (step.is_decode and step.n_tokens == step.n_seqs) else 0
+        parts = None
+        if not one_row or workspace is None:
+            splits = 1
+        elif splits is None:
+            splits = decode_splits(n, n_kv, n_heads // n_kv, v_head_dim, width)
+        if not 1 <= splits <= 64:
+            raise ValueError(f"attention: {splits} shares of a row (1 to 64)")
+        if splits > 1:
+            parts = workspace.get("attn_biased_parts", n * n_heads * splits, v_head_dim + 2, torch.float32)
         library.call(_lib(), "agave_attn_biased_mfma", ptr(q), ldq, ptr(out), ldo, ptr(gate), ldg, ptr(k_pages), ptr(v_pages),
                      ptr(table), width, ptr(base), head, n_pages, ptr(step.tok_seq), ptr(step.tok_pos), ptr(step.cu_dev), n,
                      step.n_seqs, max_rows, one_row, n_heads, n_kv, head_dim, v_head_dim, float(scale), int(window or 0),
-                     int(keep_first), bias_mode, ptr(bias) if bias_mode != BIAS_NONE else None, bias_len, ptr(sink), stream())
+                     int(keep_first), bias_mode, ptr(bias) if bias_mode != BIAS_NONE else None, bias_len, ptr(sink), splits,
+                     ptr(parts), stream())
         return
     library.call(_lib(), "agave_attn_biased_plain", dt(q), ptr(q), ldq, ptr(out), ldo, ptr(gate), ldg, ptr(k_pages),
                  ptr(v_pages), ptr(table), width, ptr(base), head, n_pages, ptr(step.tok_seq), ptr(step.tok_pos), n,

@@ -70,8 +70,8 @@ def heads_product(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, n_heads: in
     """For every token t and head h:  y[t, h * y_head + c] = sum_k w[h, c, k] * x[t, h * x_head + k]  (``w`` is
     [heads, n_out, K]); the head's next ``tail`` input elements are copied behind the product, the first
     2 * len(freq) of them rotated in pairs (i, i + len(freq)) by tok_pos[t] * freq[i]; with ``gate`` (float32
-    [N, heads * n_out]) the product is multiplied by sigmoid(gate).  Sums are 32-bit; bfloat16 rows of 16 and more
-    tokens with K a multiple of 8 run on the matrix cores."""
+    [N, heads * n_out]) the product is multiplied by sigmoid(gate).  Sums are 32-bit; bfloat16 rows with K a multiple
+    of 8 run on the matrix cores."""
     _dev(x, w, y, freq, tok_pos, gate)
     n = x.shape[0]
     ldx, ldy = _rows(x, "x"), _rows(y, "y")

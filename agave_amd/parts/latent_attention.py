@@ -129,7 +129,7 @@ class LatentAttention:
                           tok_pos=step.tok_pos)
         mixed = ws.get("latent_mixed", n, s.n_heads * s.kv_rank, x.dtype)
         attn_ops.attention(folded, mixed, None, k_pages, v_pages, table, base, 0, step, s.n_heads, 1, self.kd, s.kv_rank,
-                           s.scale, None, 0, attn_ops.BIAS_NONE, None, None, packed)
+                           s.scale, None, 0, attn_ops.BIAS_NONE, None, None, packed, workspace=ws)
         ctx = ws.get("attn_ctx", n, self.ctx, x.dtype)
         ops.heads_product(mixed, self.v_up, ctx, s.n_heads, s.kv_rank, s.v_head_dim, gate=gate)
         return self.o.forward(ctx, tag="attn_o", slices_ok=True)       # the block adds it to the residual stream

@@ -23,7 +23,7 @@ The other published shapes:
 
 Another design beside the closest Gemma 3 shape of equal size (not the default run):
 
-    python bench.py --design rilenex|gusedra [--design-size small|medium|large] [--design-layers 8]
+    python bench.py --design rilenex|gusedra|batasun [--design-size small|medium|large] [--design-layers 8]
 
 prints one JSON line with, for that decoder and for a Gemma 3 decoder of the same width, depth,
 heads and about as many weights: tokens a second of a 2,048-token prompt and of decode steps at
@@ -243,6 +243,32 @@ def gusedra_config(size: str, layers: int) -> dict:
     return {"architecture": "Gusedra", "vocab": 32768, "width": e, "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": out}
 
 
+def batasun_config(size: str, layers: int) -> dict:
+    """Of every four layers the first has latent attention with a projection of its own, the next two are state-space
+    mixers and the fourth is latent attention again that reads the first one's cached rows; every layer has the routed
+    feed-forward of the Gusedra shape beside it (16 experts of a quarter of the dense inner size, 4 of them a token,
+    and a shared expert).  Latent attention in the proportions of the published models of that kind: heads of 128
+    plain and 64 rotated elements, values of 128, a query latent of three quarters of the width, and a cached row of
+    192 + 64 numbers at the small size, 512 + 64 at the others.  State-space mixers twice as wide as the model, in
+    heads of 64 with a state of 128 per head, B and C shared by all heads."""
+    e, ff, h, _, d, _, _ = DESIGN_SIZES[size]
+    kv_rank = 192 if size == "small" else 512
+    moe = {"kind": "moe", "expert": {"ff": ff // 4, "limit": 7.0}, "shared": {"ff": ff // 4, "limit": 7.0},
+           "router": {"experts": 16, "top": 4}}
+    def latent(source):
+        m = {"heads": h, "dim": d, "rot_dim": d // 2, "vdim": d, "q_rank": 3 * e // 4, "kv_rank": kv_rank,
+             "scale": (d + d // 2) ** -0.5, "rot": {"base": 10000.0, "dims": d // 2}}
+        if source is not None:
+            m["kv_from"] = source
+        return {"type": "latent_attention", "mixer": m, "mlp": moe}
+    ssm = {"type": "mamba2", "mlp": moe,
+           "mixer": {"heads": 2 * e // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}}
+    out = []
+    for i in range(layers):
+        out.append(latent(None) if i % 4 == 0 else latent(i - 3) if i % 4 == 3 else ssm)
+    return {"architecture": "Batasun", "vocab": 32768, "width": e, "norm": {"eps": 1e-5}, "layers": out}
+
+
 def gemma_like_config(size: str, layers: int) -> dict:
     """The same width, depth and heads as a Gemma 3 decoder; its gated feed-forward has three matrices,
     so two thirds of the inner size give as many weights."""
@@ -291,8 +317,12 @@ def compare_designs(args) -> int:
     result = {"metric": f"{args.design} beside Gemma 3 at equal size ({size}, {layers} layers): tokens/s", "unit": "tokens/s",
               "dtype": "bf16", "data": "synthetic: uniform-random token ids, random weights", "sizes": DESIGN_SIZES[size],
               "peaks_measured": measured_peaks()}
-    design = {"rilenex": rilenex_config, "gusedra": gusedra_config}[args.design](size, layers)
-    for name, cfg in ((args.design, design), ("gemma3_equal_size", gemma_like_config(size, layers))):
+    makers = {"rilenex": rilenex_config, "gusedra": gusedra_config, "batasun": batasun_config}
+    runs = [(args.design, makers[args.design](size, layers))]
+    if args.design == "batasun":          # the design with routed feed-forwards and shared keys stands beside it too
+        runs.append(("gusedra_equal_size", gusedra_config(size, layers)))
+    runs.append(("gemma3_equal_size", gemma_like_config(size, layers)))
+    for name, cfg in runs:
         engine = Engine.from_random(cfg, seed=0, dtype="bfloat16", max_slots=batch, max_context=context,
                                     cache_tokens=batch * (PREFILL_LEN + 512), device="cuda:0")
         rec = {"weights_gb": round(engine.model.weight_bytes() / 1e9, 3)}
@@ -331,7 +361,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="time only the 2048-token prefill and print its record (for profiles)")
-    ap.add_argument("--design", choices=["rilenex", "gusedra"], help="measure this design beside a Gemma 3 decoder of equal size")
+    ap.add_argument("--design", choices=["rilenex", "gusedra", "batasun"], help="measure this design beside a Gemma 3 decoder of equal size")
     ap.add_argument("--design-size", default="medium", choices=sorted(DESIGN_SIZES))
     ap.add_argument("--design-layers", type=int, default=8)
     args = ap.parse_args()

@@ -41,6 +41,7 @@ class Case:
         g = torch.Generator().manual_seed(seed)
         self.H, self.G, self.d, self.vd, self.window, self.keep, self.T = H, G, d, vd, window, keep, T
         self.force_plain = False            # bfloat16 shapes that the matrix-core kernel takes run on the plain one instead
+        self.workspace, self.splits = None, None   # steps of one row: a row's pages shared among this many workgroups
         self.q = torch.randn(T, H, d, generator=g)
         self.k = torch.randn(T, G, d, generator=g)
         self.v = torch.randn(T, G, vd, generator=g)
@@ -102,7 +103,7 @@ class Case:
             out = torch.empty(hi - lo, self.H * self.vd, dtype=dtype, device=DEV)
             A.attention(dev(self.q), out, dev(self.gate) if self.gate is not None else None, kp, vp, table, base, head, step,
                         self.H, self.G, self.d, self.vd, self.scale, self.window, self.keep, self.mode, self.bias, sink,
-                        packed, force_plain=self.force_plain)
+                        packed, force_plain=self.force_plain, workspace=self.workspace, splits=self.splits)
             planner.commit(step)
             got[lo:hi] = out.float().cpu()
         if own:
@@ -128,7 +129,10 @@ SHAPES = [
     (8, 2, 128, 128, 200, 3, "table", True, True),        # the sizes of large models: the matrix cores in bfloat16
     (4, 1, 96, 48, 100, 0, "slopes", True, False),        # sizes that fill the matrix cores' steps only in part
     (34, 1, 32, 32, None, 0, "table", False, True),       # more heads to a key head than a wave has columns
-    (2, 2, 256, 256, 64, 64, "slopes", False, False),     # the largest heads
+    (2, 2, 256, 256, 64, 64, "slopes", False, False),     # the largest heads that two waves a SIMD hold
+    (16, 1, 320, 272, None, 0, "none", False, False),     # wider: one key head of cached rows for all query heads
+    (16, 1, 576, 512, None, 0, "none", False, True),      # the widest, Q in LDS
+    (3, 1, 400, 304, 130, 70, "slopes", True, False),     # the widest kernel filled in part, with a window, kept pages and sinks
 ]
 
 
@@ -144,6 +148,22 @@ def test_attention_whole_in_pieces_and_token_by_token(shape, dtype):
     if dtype == torch.bfloat16:
         c.force_plain = True
         close(c.run(cuts(T, 180, 1), dtype), ref, dtype, f"{shape} on the plain kernel")
+
+
+@pytest.mark.parametrize("shape", [SHAPES[3], SHAPES[6], SHAPES[8], SHAPES[10], SHAPES[11], SHAPES[12]])
+@pytest.mark.parametrize("splits", [None, 2, 5, 16])
+def test_a_rows_pages_shared_among_workgroups(shape, splits):
+    """Decode steps whose row's pages are shared among several workgroups (more of them than there are pages, too),
+    merged by the second kernel: sinks count once, a window's and the kept pages are found by every share."""
+    from agave_amd.ops import attention_biased as A
+    from agave_amd.parts import Workspace
+    T = 330
+    c = Case(*shape, T=T, seed=5)
+    c.rounded(torch.bfloat16)
+    ref = c.plain()
+    c.workspace, c.splits = Workspace(torch.device(DEV)), splits
+    close(c.run(cuts(T, 1, 1)[:12] + [(12, 250)] + cuts(T, 250, 1)[1:], torch.bfloat16), ref, torch.bfloat16, f"{shape} in {splits}")
+    assert 1 <= A.decode_splits(8, 1, 16, 512, 64) <= A.MAX_SPLITS and A.decode_splits(300, 4, 4, 128, 64) == 1
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
