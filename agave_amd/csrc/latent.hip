@@ -8,6 +8,11 @@
 //                    step that makes a head's values from the attention's sum over latent rows; it can copy a
 //                    head's trailing elements behind the product while rotating them, and multiply the result by
 //                    the sigmoid of a gate.
+//   latent_expand    for a prompt that starts at its first position, where every head's own keys are made from the
+//                    latent rows instead (fewer multiplications than the folded form when rows are many): the
+//                    rotated key part is put behind every head's unrotated keys, and the queries' trailing elements
+//                    are rotated in place;
+//   gate_rows        rows times the sigmoid of 32-bit logits, in place.
 //
 // Norm sums, angles, sines and the products' sums are 32-bit; T is the element type of the rows between products.
 #include "common_impl.h"
@@ -239,5 +244,81 @@ extern "C" int agave_heads_product(int dtype, const void* x, long ldx, int xs, c
         else AGAVE_CHECK(false, "heads_product: unknown dtype %d", dtype);
     }
     AGAVE_LAUNCH_CHECK("heads_product");
+    return 0;
+}
+
+
+// ------------------------------------------------------------------ every head's key row from the latent's parts
+//   kfull[t][h] = [ knope[t][h] (dim elements) | krow[t][kv_rank ..] (rot_dim elements, already rotated) ]
+//   q[t][h][dim + e], e < rot_dim: the first 2 * rot_half of them rotated in pairs (e, e + rot_half), in place
+// A workgroup per token.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_expand_kernel(T* __restrict__ q, long ldq, const T* __restrict__ knope, long ldkn,
+                                                            const T* __restrict__ krow, long ldkr, int kv_rank, T* __restrict__ kfull,
+                                                            long ldkf, const float* __restrict__ freq, int rot_half,
+                                                            const int* __restrict__ tok_pos, int heads, int dim, int rot_dim) {
+    const int t = blockIdx.x, tid = threadIdx.x, qd = dim + rot_dim;
+    const T* kn = knope + (size_t)t * ldkn;
+    const T* r = krow + (size_t)t * ldkr + kv_rank;
+    T* kf = kfull + (size_t)t * ldkf;
+    for (int i = tid; i < heads * qd; i += 256) {
+        const int h = i / qd, e = i % qd;
+        kf[i] = e < dim ? kn[(size_t)h * dim + e] : r[e - dim];
+    }
+    const float p = (float)tok_pos[t];
+    T* qr = q + (size_t)t * ldq;
+    // (a thread takes a whole pair, so nothing is read after it was written)
+    for (int i = tid; i < heads * rot_half; i += 256) {
+        const int h = i / rot_half, e = i % rot_half;
+        T* a = qr + (size_t)h * qd + dim + e;
+        float u, v;
+        turn(ld(a), ld(a + rot_half), p * freq[e], u, v);
+        st(a, u);
+        st(a + rot_half, v);
+    }
+}
+
+extern "C" int agave_latent_expand(int dtype, void* q, long ldq, const void* knope, long ldkn, const void* krow, long ldkr,
+                                   int kv_rank, void* kfull, long ldkf, const float* freq, int rot_half, const int* tok_pos,
+                                   int n_tokens, int heads, int dim, int rot_dim, hipStream_t stream) {
+    AGAVE_CHECK(n_tokens >= 0 && heads > 0 && dim > 0 && rot_dim >= 0 && kv_rank > 0 && 2 * rot_half <= rot_dim,
+                "latent_expand: bad sizes N=%d heads=%d dim=%d rot_dim=%d rotated=%d", n_tokens, heads, dim, rot_dim, 2 * rot_half);
+    AGAVE_CHECK(q && knope && krow && kfull && tok_pos && (freq || rot_half == 0), "latent_expand: null buffer");
+    AGAVE_CHECK(ldq >= (long)heads * (dim + rot_dim) && ldkf >= (long)heads * (dim + rot_dim) && ldkn >= (long)heads * dim &&
+                ldkr >= kv_rank + rot_dim, "latent_expand: a row stride is too small");
+    if (n_tokens == 0) return 0;
+    if (dtype == AGAVE_F32)
+        latent_expand_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)q, ldq, (const float*)knope, ldkn, (const float*)krow, ldkr,
+                                                                  kv_rank, (float*)kfull, ldkf, freq, rot_half, tok_pos, heads, dim, rot_dim);
+    else if (dtype == AGAVE_BF16)
+        latent_expand_kernel<bf16><<<n_tokens, 256, 0, stream>>>((bf16*)q, ldq, (const bf16*)knope, ldkn, (const bf16*)krow, ldkr,
+                                                                 kv_rank, (bf16*)kfull, ldkf, freq, rot_half, tok_pos, heads, dim, rot_dim);
+    else
+        AGAVE_CHECK(false, "latent_expand: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("latent_expand");
+    return 0;
+}
+
+// ------------------------------------------------------------------ x *= sigmoid(gate), gate in 32-bit
+template <typename T>
+__global__ void gate_rows_kernel(T* __restrict__ x, long ldx, const float* __restrict__ gate, long ldg, long total, int cols) {
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long r = idx / cols;
+        const int c = (int)(idx % cols);
+        T* at = x + r * ldx + c;
+        st(at, ld(at) * (1.0f / (1.0f + expf(-gate[r * ldg + c]))));
+    }
+}
+
+extern "C" int agave_gate_rows(int dtype, void* x, long ldx, const float* gate, long ldg, int rows, int cols, hipStream_t stream) {
+    AGAVE_CHECK(rows >= 0 && cols > 0 && ldx >= cols && ldg >= cols && x && gate, "gate_rows: bad sizes rows=%d cols=%d", rows, cols);
+    if (rows == 0) return 0;
+    const long total = (long)rows * cols;
+    long blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (dtype == AGAVE_F32) gate_rows_kernel<float><<<(int)blocks, 256, 0, stream>>>((float*)x, ldx, gate, ldg, total, cols);
+    else if (dtype == AGAVE_BF16) gate_rows_kernel<bf16><<<(int)blocks, 256, 0, stream>>>((bf16*)x, ldx, gate, ldg, total, cols);
+    else AGAVE_CHECK(false, "gate_rows: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("gate_rows");
     return 0;
 }

@@ -16,6 +16,8 @@ LIBRARY = "latent"
 
 kernels.register_signatures(LIBRARY, {
     "agave_latent_prepare": [_I, _P, _L, _P, _P, _L, _I, _P, _L, _P, _P, _L, _I, _I, _P, _I, _P, _I, _F, _P],
+    "agave_latent_expand": [_I, _P, _L, _P, _L, _P, _L, _I, _P, _L, _P, _I, _P, _I, _I, _I, _I, _P],
+    "agave_gate_rows": [_I, _P, _L, _P, _L, _I, _I, _P],
     "agave_heads_product": [_I, _P, _L, _I, _P, _P, _L, _I, _P, _L, _P, _I, _I, _P, _I, _I, _I, _I, _I, _P],
 })
 
@@ -99,3 +101,36 @@ def heads_product(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, n_heads: in
         raise ValueError(f"heads_product: a head of {k + tail} input elements is too long")
     library.call(_lib(), "agave_heads_product", dt(x), ptr(x), ldx, x_head, ptr(w), ptr(y), ldy, y_head, ptr(gate), ldg,
                  ptr(freq), rot_half, tail, ptr(tok_pos), n, n_heads, n_out, k, 1 if force_plain else 0, stream())
+
+
+def latent_expand(q: torch.Tensor, k_plain: torch.Tensor, k_row: torch.Tensor, kv_rank: int, k_full: torch.Tensor,
+                  n_heads: int, dim: int, rot_dim: int, freq: Optional[torch.Tensor], tok_pos: torch.Tensor) -> None:
+    """Every head's key row from the parts: k_full[t, h] = [k_plain[t, h] (``dim`` elements) | k_row[t, kv_rank:]
+    (``rot_dim`` elements, rotated already)]; and the last ``rot_dim`` elements of every head of ``q``
+    [N, heads * (dim + rot_dim)] are rotated in place (the first 2 * len(freq) of them, pairs (i, i + len(freq)), by
+    tok_pos[t] * freq[i])."""
+    _dev(q, k_plain, k_row, k_full, freq, tok_pos)
+    n, qd = q.shape[0], dim + rot_dim
+    ldq, ldkn, ldkr, ldkf = _rows(q, "q"), _rows(k_plain, "k_plain"), _rows(k_row, "k_row"), _rows(k_full, "k_full")
+    if tuple(q.shape) != (n, n_heads * qd) or tuple(k_full.shape) != (n, n_heads * qd) or tuple(k_plain.shape) != (n, n_heads * dim) \
+            or tuple(k_row.shape) != (n, kv_rank + rot_dim) or not (q.dtype == k_plain.dtype == k_row.dtype == k_full.dtype):
+        raise ValueError(f"latent_expand: rows of {tuple(q.shape)}, {tuple(k_plain.shape)}, {tuple(k_row.shape)} and "
+                         f"{tuple(k_full.shape)} do not hold {n_heads} heads of {dim} + {rot_dim} over a latent of {kv_rank}")
+    _i32(tok_pos, "positions", n)
+    rot_half = 0
+    if freq is not None:
+        rot_half = freq.numel()
+        _f32vec(freq, "frequencies", rot_half)
+        if 2 * rot_half > rot_dim:
+            raise ValueError(f"latent_expand: {2 * rot_half} rotated elements exceed the {rot_dim} there are")
+    library.call(_lib(), "agave_latent_expand", dt(q), ptr(q), ldq, ptr(k_plain), ldkn, ptr(k_row), ldkr, kv_rank, ptr(k_full),
+                 ldkf, ptr(freq), rot_half, ptr(tok_pos), n, n_heads, dim, rot_dim, stream())
+
+
+def gate_rows(x: torch.Tensor, gate: torch.Tensor) -> None:
+    """x *= sigmoid(gate) in place; ``gate`` is float32 of ``x``'s shape (column slices are fine)."""
+    _dev(x, gate)
+    n, cols = x.shape
+    ldx = _rows(x, "x")
+    ldg = _f32rows(gate, "gate", n, cols)
+    library.call(_lib(), "agave_gate_rows", dt(x), ptr(x), ldx, ptr(gate), ldg, n, cols, stream())

@@ -138,6 +138,34 @@ def test_batches_of_unequal_requests_and_slots_used_again(models, dtype):
     assert all(g.pool.n_free == g.pool.n_pages for g in eng.cache.groups)
 
 
+def test_prompts_from_their_first_position_make_every_heads_keys(models):
+    """In bfloat16, with head sizes the matrix cores take, a step of prompts that all start at position 0 runs the
+    attention over every head's own keys and values instead of the cached latent rows; its pieces and the decoding
+    after it read the latent rows.  Unequal prompts together (one shorter than a page, one ending on a page's border),
+    a reader of another layer's rows among the layers, and the same prompts in pieces, against the plain logits."""
+    cfg, w, folder = models("even", decided=True)
+    eng = engine(folder, "bfloat16", max_slots=3, max_context=512)
+    latent = [b.mixer for b in eng.model.blocks if hasattr(b.mixer, "fresh_prompt")]
+    assert len(latent) == 2 and all(m.fresh_ok for m in latent)
+    calls = []
+    for m in latent:
+        def counted(*a, inner=m.fresh_prompt, **k):
+            calls.append(1)
+            return inner(*a, **k)
+        m.fresh_prompt = counted
+    reqs = [U.random_tokens(n, cfg["vocab"], 40 + n) for n in (150, 40, 128)]
+    refs = [P.forward(cfg, w, r) for r in reqs]
+    for r, o in zip(refs, U.run_batched(eng, reqs, (141, 33, 128))):
+        close(o, r, "bfloat16", "prompts together, then decoded")
+    assert len(calls) == 2
+    eng.prefill_chunk = 70                                  # the first piece from position 0, the others behind it
+    close(U.run_whole(eng, reqs[0]), refs[0], "bfloat16", "pieces of 70")
+    assert len(calls) == 4
+    eng.prefill_chunk = 0
+    close(U.run_tail(eng, reqs[2], 100), refs[2], "bfloat16", "28 tokens (the latent rows' form), then decoded")
+    assert len(calls) == 4
+
+
 def test_the_cache_as_the_mixers_asked(models):
     cfg, w, folder = models("mixed")
     eng = engine(folder, "float32")

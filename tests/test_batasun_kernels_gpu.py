@@ -94,6 +94,30 @@ def test_products_per_head_with_trailing_elements_and_a_gate(dtype, n, heads, K,
             assert rel(y2.view(n, heads, n_out), prod * torch.sigmoid(gate.to(F64)).view(n, heads, n_out)) < tol, plain
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads, dim, rot_dim, rot, kv_rank", [(4, 32, 16, 16, 48), (3, 10, 6, 4, 7), (1, 128, 64, 64, 512), (5, 8, 0, 0, 16)])
+def test_every_heads_key_row_from_the_parts_and_the_gate(dtype, heads, dim, rot_dim, rot, kv_rank):
+    from agave_amd.ops import latent as L
+    n, qd = 37, dim + rot_dim
+    g = torch.Generator().manual_seed(dim)
+    pos = [(11 * t) % 500 for t in range(n)]
+    q = torch.randn(n, heads * qd, generator=g).to(dtype)
+    k_plain = torch.randn(n, heads * dim, generator=g).to(dtype)
+    k_row = torch.randn(n, kv_rank + rot_dim, generator=g).to(dtype)
+    freq = torch.tensor([90.0 ** (-2.0 * e / rot) for e in range(rot // 2)], dtype=torch.float32, device=DEV) if rot else None
+    qd_, k_full = q.to(DEV), torch.empty(n, heads * qd, dtype=dtype, device=DEV)
+    L.latent_expand(qd_, k_plain.to(DEV), k_row.to(DEV), kv_rank, k_full, heads, dim, rot_dim, freq, Positions(pos).tok_pos)
+    q64 = q.to(F64).view(n, heads, qd)
+    want_q = torch.cat([q64[..., :dim], P.rotate(q64[..., dim:], pos, 90.0, rot) if rot else q64[..., dim:]], -1)
+    want_k = torch.cat([k_plain.to(F64).view(n, heads, dim), k_row.to(F64)[:, None, kv_rank:].expand(n, heads, rot_dim)], -1)
+    assert torch.equal(k_full.cpu().to(F64).view(n, heads, qd), want_k)
+    assert rel(qd_.view(n, heads, qd), want_q) < (4e-4 if dtype == torch.float32 else 8e-3)
+    wide = torch.randn(n, heads * qd + 3, generator=g) * 3
+    x = q.to(DEV).clone()
+    L.gate_rows(x, wide.to(DEV)[:, 1:1 + heads * qd])
+    assert rel(x, q.to(F64) * torch.sigmoid(wide.to(F64)[:, 1:1 + heads * qd])) < (1e-5 if dtype == torch.float32 else 5e-3)
+
+
 # ---------------------------------------------------------------- the state-space recurrence
 def run_state_space(t, sizes, plan_rows, vectors):
     from agave_amd.cache import StateNeed
