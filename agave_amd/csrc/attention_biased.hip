@@ -447,35 +447,77 @@ __global__ __launch_bounds__((KS > 8 || VB > 16) ? 256 : 512) void attn_biased_m
         }
         // scores of the page's four key blocks
         f32x4_t s[NC][4];
+        if constexpr (KS > 9 && !QL) {
+            // A long head: the page's 4 KS key operands in chunks of four, a chunk asked for while the one before it is
+            // multiplied (two sets of registers that take turns).  The compiler is told not to move anything across
+            // a chunk's border: left alone it asks for everything at once and runs out of registers, and a loop that
+            // waits for every chunk before it asks for the next is a chain of round trips to memory.
+            constexpr int C = 4, NCH = (4 * KS + C - 1) / C;
+            frag16 kbuf[2][C];
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb) {
-            // (a whole operand in one load of a kilobyte; steps past the head's end read step 0 again and are emptied)
-            // (a long head's steps come in two or three batches, so that no more than six or nine operands wait in registers; the
-            // compiler is told not to move anything across the batches' border, or it asks for all of them at once)
-            constexpr int KCH = KS > 12 ? 6 : KS > 9 ? (KS + 1) / 2 : KS;
+            for (int cb = 0; cb < NC; ++cb)
 #pragma unroll
-            for (int cb = 0; cb < NC; ++cb) s[cb][kb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                for (int kb = 0; kb < 4; ++kb) s[cb][kb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int k0 = 0; k0 < KS; k0 += KCH) {
-                frag16 kf[KCH];
+            for (int ch = -1; ch < NCH; ++ch) {
+                if (ch + 1 < NCH) {
 #pragma unroll
-                for (int kk = 0; kk < KCH; ++kk) {
-                    const int ks = k0 + kk;
-                    const u32x4_t got = kt[(kb * ksl + (ks < ksl ? ks : 0)) * 64 + lane];
-                    kf[kk].r = ks < ksl ? got : u32x4_t{0u, 0u, 0u, 0u};
-                }
-#pragma unroll
-                for (int cb = 0; cb < NC; ++cb) {
-#pragma unroll
-                    for (int kk = 0; kk < KCH; ++kk)
-                        if (k0 + kk < KS) {
-                            frag16 qv;
-                            if constexpr (QL) qv.r = qs[(k0 + kk) * 64 + lane];
-                            else qv = qf[cb][k0 + kk];
-                            s[cb][kb] = mfma_16x16x32(kf[kk], qv, s[cb][kb]);
+                    for (int i = 0; i < C; ++i) {
+                        const int e = (ch + 1) * C + i;
+                        if (e < 4 * KS) {
+                            const int kb = e / KS, ks = e % KS;
+                            const u32x4_t got = kt[(kb * ksl + (ks < ksl ? ks : 0)) * 64 + lane];
+                            kbuf[(ch + 1) & 1][i].r = ks < ksl ? got : u32x4_t{0u, 0u, 0u, 0u};
                         }
+                    }
                 }
-                if constexpr (KS > 9) __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (ch >= 0) {
+#pragma unroll
+                    for (int i = 0; i < C; ++i) {
+                        const int e = ch * C + i;
+                        if (e < 4 * KS) {
+                            const int kb = e / KS, ks = e % KS;
+#pragma unroll
+                            for (int cb = 0; cb < NC; ++cb) {
+                                s[cb][kb] = mfma_16x16x32(kbuf[ch & 1][i], qf[cb][ks], s[cb][kb]);
+                            }
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < 4; ++kb) {
+                // (a whole operand in one load of a kilobyte; steps past the head's end read step 0 again and are
+                // emptied.  The longest heads, which have no registers left for a second set of operands, take their
+                // steps in three batches that wait for each other.)
+                constexpr int KCH = QL ? 6 : KS;
+#pragma unroll
+                for (int cb = 0; cb < NC; ++cb) s[cb][kb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int k0 = 0; k0 < KS; k0 += KCH) {
+                    frag16 kf[KCH];
+#pragma unroll
+                    for (int kk = 0; kk < KCH; ++kk) {
+                        const int ks = k0 + kk;
+                        const u32x4_t got = kt[(kb * ksl + (ks < ksl ? ks : 0)) * 64 + lane];
+                        kf[kk].r = ks < ksl ? got : u32x4_t{0u, 0u, 0u, 0u};
+                    }
+#pragma unroll
+                    for (int cb = 0; cb < NC; ++cb) {
+#pragma unroll
+                        for (int kk = 0; kk < KCH; ++kk)
+                            if (k0 + kk < KS) {
+                                frag16 qv;
+                                if constexpr (QL) qv.r = qs[(k0 + kk) * 64 + lane];
+                                else qv = qf[cb][QL ? 0 : k0 + kk];
+                                s[cb][kb] = mfma_16x16x32(kf[kk], qv, s[cb][kb]);
+                            }
+                    }
+                    if constexpr (QL) __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
         // Scale, bias, mask and softmax, a column block at a time, in the base-2 domain (scale, slopes, table and
@@ -546,6 +588,38 @@ __global__ __launch_bounds__((KS > 8 || VB > 16) ? 256 : 512) void attn_biased_m
             if (whole) scores(IntC<1>{}, IntC<0>{}); else scores(IntC<0>{}, IntC<0>{});
         }
         // O^T = O^T alpha + V^T P^T
+        if constexpr (VB > 16 && !QL) {
+            // (wide values: two blocks' operands at a time, the next two asked for while these are multiplied)
+            constexpr int VG = 2, NVG = VB / VG;
+            frag16 vbuf[2][VG][2];
+#pragma unroll
+            for (int gi = -1; gi < NVG; ++gi) {
+                if (gi + 1 < NVG) {
+#pragma unroll
+                    for (int j = 0; j < VG; ++j) {
+                        const int nb = (gi + 1) * VG + j, nbl = 16 * nb < vd ? nb : 0;     // (a block past the value size reads the first again)
+#pragma unroll
+                        for (int h2 = 0; h2 < 2; ++h2) vbuf[(gi + 1) & 1][j][h2].r = vt[(nbl * 2 + h2) * 64 + lane];
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (gi >= 0) {
+#pragma unroll
+                    for (int j = 0; j < VG; ++j) {
+                        const int nb = gi * VG + j;
+                        if (16 * nb < vd) {
+#pragma unroll
+                            for (int cb = 0; cb < NC; ++cb) {
+                                o[cb][nb] *= alpha[cb];
+                                o[cb][nb] = mfma_16x16x32(vbuf[gi & 1][j][0], pf[cb][0], o[cb][nb]);
+                                o[cb][nb] = mfma_16x16x32(vbuf[gi & 1][j][1], pf[cb][1], o[cb][nb]);
+                            }
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        } else {
 #pragma unroll
         for (int nb = 0; nb < VB; ++nb) {
             if (16 * nb < vd) {
@@ -564,9 +638,10 @@ __global__ __launch_bounds__((KS > 8 || VB > 16) ? 256 : 512) void attn_biased_m
                     o[cb][nb] = mfma_16x16x32(vf[1], pf[cb][1], o[cb][nb]);
                 }
             }
-            if constexpr (VB > 16) {                    // (four blocks' value operands at a time, see above)
+            if constexpr (QL) {                         // (four blocks' value operands at a time, see the keys)
                 if ((nb & 3) == 3) __builtin_amdgcn_sched_barrier(0);
             }
+        }
         }
     };
 
@@ -663,9 +738,13 @@ __global__ __launch_bounds__((KS > 8 || VB > 16) ? 256 : 512) void attn_biased_m
             l[0] = l[0] * a1 + l2 * a2;
             m[0] = m_new;
 #pragma unroll
-            for (int nb = 0; nb < VB; ++nb)
+            for (int nb = 0; nb < VB; ++nb) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) o[0][nb][e] = o[0][nb][e] * a1 + other[32 + (16 * nb + 4 * g + (e ^ (g & 1))) * 16 + c] * a2;
+                if constexpr (VB > 16) {                // (or all of the other wave's row is read before any of it is used)
+                    if ((nb & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+                }
+            }
         }
         if (splits > 1) {
             // this workgroup's share of the row: reference, sum and the unnormalised sums over the values

@@ -173,17 +173,25 @@ __global__ __launch_bounds__(256) void heads_product_mfma_kernel(HeadsProductArg
     f32x4_t acc[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < K; k0 += 32) {
-        // (loads without conditions, from inside the row; a lane past the row's end reads its start and is emptied)
-        const bool in = k0 + 8 * g < K;
-        const int at = in ? k0 : -8 * g;
-        frag16 a, b[4];
-        a.u = *reinterpret_cast<const uint4*>(arow + at);
+    // four steps along K at a time: their loads leave together (without conditions, from inside the row; a lane past the
+    // row's end reads its start and is emptied), so a product is a few round trips to memory and not one per step
+    for (int k0 = 0; k0 < K; k0 += 128) {
+        frag16 a[4], b[4][4];
+        bool in[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) b[j].u = *reinterpret_cast<const uint4*>(brow[j] + at);
-        if (!in) a.u = make_uint4(0, 0, 0, 0);
+        for (int u = 0; u < 4; ++u) {
+            in[u] = k0 + 32 * u + 8 * g < K;
+            const int at = in[u] ? k0 + 32 * u : -8 * g;
+            a[u].u = *reinterpret_cast<const uint4*>(arow + at);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = mfma_16x16x32(a, b[j], acc[j]);
+            for (int j = 0; j < 4; ++j) b[u][j].u = *reinterpret_cast<const uint4*>(brow[j] + at);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (!in[u]) a[u].u = make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = mfma_16x16x32(a[u], b[u][j], acc[j]);
+        }
     }
     // D[j]: the lane holds tokens row0 + 4 g + e4, column col0 + 16 j + c
 #pragma unroll

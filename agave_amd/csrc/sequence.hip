@@ -1021,14 +1021,14 @@ extern "C" int agave_head_norm_gate(int dtype, const float* o, long ldo_in, cons
 
 // ------------------------------------------------------------------ a gate, then a norm in equal parts of the row
 //   g = y * silu(z);  out = g / sqrt(mean over the part (g^2) + eps) * w     (w is [parts * size])
-// A workgroup per (token, part), of one to four waves by the part's size; a thread keeps up to eight gated values in
+// A workgroup per (token, part), of one to four waves by the part's size; a thread keeps up to sixteen gated values in
 // registers between the sum of squares and the output (longer parts are computed twice).
 template <typename T>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ y, long ldy, const float* __restrict__ z,
                                                                long ldz, const float* __restrict__ w, T* __restrict__ out, long ldo,
                                                                int parts, int size, float eps) {
     __shared__ float red[8];
-    constexpr int KEEP = 8;
+    constexpr int KEEP = 16;
     const int t = blockIdx.x / parts, g = blockIdx.x % parts, tid = threadIdx.x, nt = blockDim.x;
     const float* yr = y + (size_t)t * ldy + (size_t)g * size;
     const float* zr = z + (size_t)t * ldz + (size_t)g * size;
