@@ -39,7 +39,7 @@ extern "C" int agave_embed_scale(int dtype, const int* tokens, const void* table
 // ------------------------------------------------------------------ residual + norms
 //   r = rows ? rows[i] : i                       (row of h and of branch)
 //   if branch: h[r] += post_gain ? rmsnorm(branch[r]) * post_gain : branch[r]
-//   if out:    out[i] = rmsnorm(h[r]) * pre_gain
+//   if out:    out[i] = pre_gain ? rmsnorm(h[r]) * pre_gain : h[r]      (a layer without a norm in front of a sublayer)
 // Gains are 32-bit and already hold the "+1" where the architecture has it.
 template <typename T>
 __global__ void residual_norm_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb, int n_parts,
@@ -85,11 +85,15 @@ __global__ void residual_norm_kernel(float* __restrict__ h, const T* __restrict_
             ss_h += hv * hv;
         }
     }
-    if (out) {
+    if (out && pre_gain) {
         ss_h = block_sum(ss_h, red);
         const float inv = 1.0f / sqrtf(ss_h / (float)e + pre_eps);
         T* o = out + (size_t)i * ldo;
         for (int c = threadIdx.x; c < e; c += blockDim.x) st(o + c, hr[c] * inv * pre_gain[c]);
+    } else if (out) {
+        __syncthreads();                                // (the row was written by other threads of the workgroup)
+        T* o = out + (size_t)i * ldo;
+        for (int c = threadIdx.x; c < e; c += blockDim.x) st(o + c, hr[c]);
     }
 }
 
@@ -138,7 +142,7 @@ __global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __rest
     bool in[VPT];
     // a gain that is not there is read from the row itself and not used
     const float* g1p = (branch && post_gain) ? post_gain : hr;
-    const float* g2p = out ? pre_gain : hr;
+    const float* g2p = (out && pre_gain) ? pre_gain : hr;
 #pragma unroll
     for (int v = 0; v < VPT; ++v) {
         const int c = (threadIdx.x + v * blockDim.x) * 4;
@@ -205,7 +209,12 @@ __global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __rest
         for (int v = 0; v < VPT; ++v)
             if (in[v]) *reinterpret_cast<float4*>(hr + col[v]) = hv[v];
     }
-    if (out) {
+    if (out && !pre_gain) {                             // the rows as they are, rounded to the output's type
+        T* o = out + (size_t)i * ldo;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v)
+            if (in[v]) store4(o + col[v], hv[v]);
+    } else if (out) {
         float ss = 0.f;
 #pragma unroll
         for (int v = 0; v < VPT; ++v) ss += sumsq(in[v], hv[v]);
@@ -272,7 +281,6 @@ extern "C" int agave_residual_norm(int dtype, float* h, const void* branch, long
     AGAVE_CHECK(n_rows >= 0 && e > 0, "residual_norm: bad sizes rows=%d e=%d", n_rows, e);
     AGAVE_CHECK(h != nullptr, "residual_norm: residual stream is null");
     AGAVE_CHECK(!(h_src && rows), "residual_norm: rows are gathered from the residual stream itself, not from another source");
-    AGAVE_CHECK(!out || pre_gain, "residual_norm: output without its gain");
     AGAVE_CHECK(!branch || ldb >= e, "residual_norm: branch row stride %ld < %d", ldb, e);
     AGAVE_CHECK(!out || ldo >= e, "residual_norm: output row stride %ld < %d", ldo, e);
     AGAVE_CHECK(!(rows && branch), "residual_norm: row gather with a branch is not supported");

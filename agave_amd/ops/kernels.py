@@ -133,8 +133,8 @@ def embed_scale(tokens: torch.Tensor, table: torch.Tensor, scale: float, out: to
 def residual_norm(h: torch.Tensor, branch: Optional[torch.Tensor], post_gain: Optional[torch.Tensor],
                   post_eps: float, out: Optional[torch.Tensor], pre_gain: Optional[torch.Tensor],
                   pre_eps: float, rows: Optional[torch.Tensor] = None, src: Optional[torch.Tensor] = None) -> None:
-    """If ``branch``: h += rmsnorm(branch) * post_gain.  If ``out``: out = rmsnorm(h) * pre_gain.
-    ``rows`` (int32) picks the rows of ``h`` that ``out`` is computed for.  A three-dimensional
+    """If ``branch``: h += rmsnorm(branch) * post_gain.  If ``out``: out = rmsnorm(h) * pre_gain, or the rows of h
+    as they are, rounded to ``out``'s type, where ``pre_gain`` is None.  ``rows`` (int32) picks the rows of ``h`` that ``out`` is computed for.  A three-dimensional
     float32 ``branch`` [slices, rows, hidden] stands for the sum of its slices (a product that was
     shared out along its columns).  ``src``: the residual rows are read from this tensor and
     written to ``h`` (a kernel that could not update the stream in place left it there)."""

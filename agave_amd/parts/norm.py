@@ -110,7 +110,16 @@ class NormedRows:
 
 def rows_as_they_are(h: torch.Tensor, pending: Pending, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
     """What stands where a norm would for a model without one: the pending branch is added and
-    the (chosen) rows of ``h`` are handed on, rounded to ``out``'s element type."""
+    the (chosen) rows of ``h`` are handed on, rounded to ``out``'s element type.  One kernel where the
+    branch's norm is an RMS norm (or none) and all rows are wanted, as with a norm in front."""
+    branch, post, base = unpack_pending(pending)
+    fused = rows is None and branch is not None and (post is None or isinstance(post, RmsNorm))
+    if fused and branch.dim() == 2 and branch.dtype != out.dtype:
+        fused = False
+    if fused:
+        kernels.residual_norm(h, branch, post.gain if post is not None else None, post.eps if post is not None else 0.0,
+                              out, None, 0.0, None, src=base)
+        return
     add_branch(h, pending)
     kernels.gather_rows(h, rows, out)
 
