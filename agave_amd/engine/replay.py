@@ -98,12 +98,18 @@ def tokens_held(records: Sequence[dict]) -> int:
     return most
 
 
+MAX_LIVE = 256          # the most requests a replay holds at a time
+
+
 class Replay:
     def __init__(self, model_dir: str, dtype: str, max_tokens: int):
         pages = (int(max_tokens) + PAGE - 1) // PAGE
-        # every live request holds at least one page, so there are never more requests than pages
-        self.engine = Engine.from_folder(model_dir, dtype=dtype, max_slots=pages,
-                                         max_context=pages * PAGE, cache_tokens=pages * PAGE, will_sample=False)
+        # ``max_tokens`` counts tokens, and a request holds whole pages: every live request may waste up to a page less
+        # one token, so the pool gets a page more per slot than the tokens alone would fill.  Every live request
+        # holds at least one token, so there are never more requests than tokens (nor, for the slots' sake, than 256).
+        slots = max(1, min(int(max_tokens), MAX_LIVE))
+        self.engine = Engine.from_folder(model_dir, dtype=dtype, max_slots=slots, max_context=pages * PAGE,
+                                         cache_tokens=(pages + slots) * PAGE, will_sample=False)
         self.slot_of: Dict[str, int] = {}
 
     def run_step(self, entries: Sequence[dict], end: Sequence[str]) -> Optional[np.ndarray]:

@@ -293,7 +293,7 @@ def test_command_line_and_trace_replay(models, tmp_path):
     firsts = [(8, 3, 78), (1, 59)]
     records, where = U.trace_steps_batched(batches, firsts)
     for dtype in ("float32", "bfloat16"):
-        steps = U.run_trace_tool(folder, dtype, records, str(tmp_path / dtype), 256, cfg["vocab"])
+        steps = U.run_trace_tool(folder, dtype, records, str(tmp_path / dtype), 153, cfg["vocab"])      # the tokens held, counted one by one: three requests need four pages
         for bi, reqs in enumerate(batches):
             for i, r in enumerate(reqs):
                 got = torch.from_numpy(np.stack([steps[s][row] for s, row in where[(bi, i)]]))

@@ -167,7 +167,7 @@ def test_state_space_whole_pieces_and_tokens(H, G, N, dv):
 def test_state_space_step_sizes_without_a_clamp_and_a_write_far_back():
     """Step sizes from almost nothing to dozens (softplus of -20 to 40, neither clamped); and with a decay rate of
     almost nothing what token 3 wrote is read 600 tokens later among small writes, while a fast rate forgets it."""
-    H, G, N, dv, T = 1, 1, 8, 4, 640
+    H, G, N, dv, T = 1, 1, 8, 4, 650
     g = torch.Generator().manual_seed(5)
     for a_log, kept in ((-12.0, True), (1.0, False)):
         t = {"xs": 0.01 * torch.randn(T, dv, generator=g), "B": torch.zeros(T, N), "C": torch.zeros(T, N),
