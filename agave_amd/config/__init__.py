@@ -1,12 +1,13 @@
 """Typed configurations and the architecture registry."""
 from .batasun import BatasunConfig
+from .duperax import DuperaxConfig
 from .errors import ConfigError, UnsupportedArchitecture
 from .gemma3 import Gemma3Config
 from .gusedra import GusedraConfig
 from .registry import (Architecture, architectures, find_architecture, load_config,
                        read_config_json, register_architecture)
 from .rilenex import RilenexConfig
-from .spec import (AttentionSpec, BiasedAttentionSpec, LatentAttentionSpec, Mamba2Spec, RoutedFfnSpec, ScoreBiasSpec, DenseFfnSpec, FeedForwardSpec, GatedDeltaSpec, GatedFfnSpec, Hgrn2Spec, LayerSpec,
+from .spec import (RglruSpec, StreamMixSpec, AttentionSpec, BiasedAttentionSpec, LatentAttentionSpec, Mamba2Spec, RoutedFfnSpec, ScoreBiasSpec, DenseFfnSpec, FeedForwardSpec, GatedDeltaSpec, GatedFfnSpec, Hgrn2Spec, LayerSpec,
                    MixerSpec, ModelSpec, NormSpec, ParallelMixerSpec, PositionSpec, RunEntry, TalkingAttentionSpec)
 
 register_architecture(Architecture(
@@ -33,8 +34,14 @@ register_architecture(Architecture(
     parse=BatasunConfig.from_dict,
     spec=lambda cfg, names=None: cfg.model_spec(names)))
 
+register_architecture(Architecture(
+    name=DuperaxConfig.architecture,
+    model_types=("duperax",),
+    parse=DuperaxConfig.from_dict,
+    spec=lambda cfg, names=None: cfg.model_spec(names)))
+
 __all__ = [
-    "ConfigError", "UnsupportedArchitecture", "Gemma3Config", "RilenexConfig", "GusedraConfig", "BatasunConfig", "LatentAttentionSpec", "Mamba2Spec", "BiasedAttentionSpec", "RoutedFfnSpec", "ScoreBiasSpec", "Architecture", "architectures",
+    "DuperaxConfig", "RglruSpec", "StreamMixSpec", "ConfigError", "UnsupportedArchitecture", "Gemma3Config", "RilenexConfig", "GusedraConfig", "BatasunConfig", "LatentAttentionSpec", "Mamba2Spec", "BiasedAttentionSpec", "RoutedFfnSpec", "ScoreBiasSpec", "Architecture", "architectures",
     "find_architecture", "load_config", "read_config_json", "register_architecture",
     "AttentionSpec", "FeedForwardSpec", "GatedFfnSpec", "LayerSpec", "MixerSpec", "ModelSpec",
     "NormSpec", "PositionSpec", "RunEntry", "TalkingAttentionSpec", "GatedDeltaSpec", "Hgrn2Spec",

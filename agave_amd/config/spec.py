@@ -29,11 +29,20 @@ class NormSpec:
 @dataclass(frozen=True)
 class PositionSpec:
     """A position encoding applied to queries and keys inside a mixer."""
-    kind: str                      # "rope" | "none"
+    kind: str                      # "rope" | "rope_yarn" | "none"
     rotary_dim: int = 0
     theta: float = 0.0
     factor: float = 1.0            # linear scaling: positions are divided by it
     interleaved: bool = False      # the rotated pairs are (2i, 2i+1) instead of (i, i + rotary_dim/2)
+    # "rope_yarn": pair i's frequency f_i = theta^(-2i/rotary_dim) becomes f_i / yarn_factor * r_i + f_i (1 - r_i) with
+    # r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), lo = max(floor(d(yarn_fast)), 0), hi = min(ceil(d(yarn_slow)),
+    # rotary_dim - 1), d(t) = rotary_dim ln(yarn_original / (2 pi t)) / (2 ln theta); sine and cosine are multiplied by
+    # yarn_magnitude_slope ln(yarn_factor) + 1
+    yarn_factor: float = 1.0
+    yarn_original: int = 0
+    yarn_fast: float = 32.0
+    yarn_slow: float = 1.0
+    yarn_magnitude_slope: float = 0.1
 
 
 @dataclass(frozen=True)
@@ -109,7 +118,13 @@ class BiasedAttentionSpec(MixerSpec):
     """Softmax attention without a rotation whose scores get a bias by distance, with keys and values of
     different sizes, a window, first positions that stay visible, an optional sink in the softmax's
     denominator and an optional sigmoid gate on the concatenated heads.  Without ``k_proj`` and ``v_proj``
-    the mixer has no keys and values of its own and reads the memory its run-order entry names."""
+    the mixer has no keys and values of its own and reads the memory its run-order entry names.
+
+    Optional besides: biases on the q, k and v products; an RMS norm over the whole row of q and of k (all heads side by
+    side, one weight per element; ``q_row_norm``, ``k_row_norm``), before a rotation of the heads' first elements
+    (``position``); a cap on the scaled scores, ``softcap * tanh(score / softcap)``, before the bias; and chunks
+    instead of (or besides) a window: a query sees only keys of its own chunk of ``chunk`` positions, counted from the
+    sequence's first."""
     hidden: int = 0
     n_heads: int = 0
     n_kv_heads: int = 0
@@ -125,6 +140,14 @@ class BiasedAttentionSpec(MixerSpec):
     k_proj: str = ""
     v_proj: str = ""
     o_proj: str = ""
+    q_bias: str = ""               # names of the products' bias vectors; "": none
+    k_bias: str = ""
+    v_bias: str = ""
+    q_row_norm: Optional[NormSpec] = None      # RMS norm over the whole q row [heads * head_dim]
+    k_row_norm: Optional[NormSpec] = None      # over the whole k row [kv heads * head_dim]
+    position: PositionSpec = PositionSpec("none")
+    softcap: float = 0.0           # > 0: score <- softcap * tanh(score / softcap)
+    chunk: Optional[int] = None    # None: no chunks; C: only keys j with j // C == i // C
 
 
 @dataclass(frozen=True)
@@ -233,6 +256,33 @@ class Hgrn2Spec(MixerSpec):
 
 
 @dataclass(frozen=True)
+class RglruSpec(MixerSpec):
+    """A gated linear recurrence per channel (state [width]) beside a GELU branch.
+
+    ``y = gelu_tanh(y_proj x + y_bias)``; ``u = conv(x_proj x + x_bias)`` (a short causal convolution per channel with a
+    bias, no activation); in each of ``blocks`` equal parts b of the channels ``r = sigmoid(r_gate[b] u_b + r_bias[b])``
+    and ``g = sigmoid(i_gate[b] u_b + i_bias[b])``; ``a = exp(-decay_scale r softplus(lam))``;
+    ``S <- a S + sqrt(1 - a^2) g u`` from S = 0; the result is ``o_proj (S y)``."""
+    hidden: int = 0
+    width: int = 0
+    blocks: int = 1
+    conv_taps: int = 1
+    decay_scale: float = 8.0
+    y_proj: str = ""
+    y_bias: str = ""
+    x_proj: str = ""
+    x_bias: str = ""
+    conv: str = ""                 # [width, taps], the last column is the current token's
+    conv_bias: str = ""
+    r_gate: str = ""               # [blocks, width / blocks, width / blocks], [out, in] inside a block
+    r_bias: str = ""               # [blocks, width / blocks]
+    i_gate: str = ""
+    i_bias: str = ""
+    lam: str = ""                  # [width]
+    o_proj: str = ""
+
+
+@dataclass(frozen=True)
 class ParallelMixerSpec(MixerSpec):
     """Mixers side by side on the same input; the result is the sum of ``scales[i] * branches[i]``."""
     branches: Tuple[MixerSpec, ...] = ()
@@ -284,7 +334,10 @@ class RoutedFfnSpec(FeedForwardSpec):
 
     ``score="softmax_top"`` instead: the router's logits plus ``correction`` (a bias of the logits here) decide, the
     ``top`` largest are chosen, and the weights are the softmax over the chosen logits alone, times ``route_scale``
-    (no groups).  ``act_limit`` and ``act_alpha`` are the activation's numbers where it has some
+    (no groups).  ``score="sigmoid"``: the scores are ``sigmoid`` of the logits, each on its own; choice and groups as
+    with ``softmax_all``.  ``group_top``: a group counts by the sum of its this many largest scores + correction (1: by
+    its largest).  ``normalise``: the chosen experts' weights are divided by their sum + 1e-20 (before ``route_scale``).
+    ``act_limit`` and ``act_alpha`` are the activation's numbers where it has some
     (``swish_clamped``, see :class:`GatedFfnSpec`)."""
     hidden: int = 0
     intermediate: int = 0          # of every expert
@@ -302,7 +355,9 @@ class RoutedFfnSpec(FeedForwardSpec):
     up_name: str = "up"
     down_name: str = "down"
     shared: Optional[GatedFfnSpec] = None
-    score: str = "softmax_all"     # | "softmax_top"
+    score: str = "softmax_all"     # | "softmax_top" | "sigmoid"
+    group_top: int = 1
+    normalise: bool = False
     shared_gate: str = ""          # [1, hidden]; "": the shared expert is added as it is
     act_limit: float = 0.0
     act_alpha: float = 1.0
@@ -316,6 +371,9 @@ class LayerSpec:
                     h += post_ffn_norm(ffn(pre_ffn_norm(h)))
     ``"prenorm"``:  the same without the two post norms.
     ``"postnorm"``: h += post_mixer_norm(mixer(h));  h += post_ffn_norm(ffn(h)): the sublayers read the stream itself.
+    ``"streams"``:  the residual is ``ModelSpec.streams`` rows x_1 .. x_S per token; a sublayer reads
+                    u = sum_s read[s] x_s, computes y = sublayer(pre_norm(u)), and writes, all streams at once,
+                    x_t <- sum_s mix[s, t] x_s + write[t] y (``mixer_streams``, ``ffn_streams``).
     """
     kind: str
     mixer: MixerSpec
@@ -324,6 +382,17 @@ class LayerSpec:
     post_mixer_norm: Optional[NormSpec] = None
     pre_ffn_norm: Optional[NormSpec] = None
     post_ffn_norm: Optional[NormSpec] = None
+    mixer_streams: Optional["StreamMixSpec"] = None
+    ffn_streams: Optional["StreamMixSpec"] = None
+
+
+@dataclass(frozen=True)
+class StreamMixSpec:
+    """How one sublayer reads and writes several residual streams (tensor names)."""
+    streams: int
+    read: str                      # [streams]: the sublayer's input is sum_s read[s] x_s
+    write: str                     # [streams]: stream t receives write[t] times the sublayer's result
+    mix: str                       # [streams, streams], indexed [from, to]: the streams are mixed as the result is added
 
 
 @dataclass(frozen=True)
@@ -360,6 +429,9 @@ class ModelSpec:
     logit_scale: float = 1.0
     logit_softcap: float = 0.0
     embed_norm: Optional[NormSpec] = None    # a norm on the embedding rows before the first layer
+    # > 0: the residual is this many streams per token (layers of kind "streams"), all equal to the embedding row at
+    # the start; their sum enters the final norm.  0: one stream, the ordinary residual sum.
+    streams: int = 0
     extra: Dict[str, object] = field(default_factory=dict)
 
     def default_order(self) -> List[RunEntry]:

@@ -6,6 +6,8 @@
 //   * the bias: none; a slope per head, score -= slope_h * (p - j); or a table per head over
 //     distances, score += table[h][min(p - j, len - 1)] (the host folds any bucketing of
 //     distances into the table);
+//   * chunks: a query sees only keys of its own chunk of C positions (j / C == p / C), chunks counted from the
+//     sequence's first position; a cap on the scaled scores, cap * tanh(scale q.k / cap), before the bias;
 //   * a sink per head: exp(sink_h) is added to the softmax's denominator, with no key or value;
 //   * a gate on the output rows: out *= sigmoid(gate), element by element.
 // Scores, bias, softmax and the sums over values are 32-bit in every element type.
@@ -93,6 +95,79 @@ extern "C" int agave_kv_append_rows(int dtype, const void* k, long ldk, const vo
     return 0;
 }
 
+// ------------------------------------------------------------------ q and k rows before they meet
+// 32-bit rows of a step's q, k and v (the projections' results, side by side or apart) become the rows the attention
+// reads and the cache holds: q and k are divided by the root mean square of their whole row (all heads side by side)
+// and multiplied by a weight per element where the mixer has such a norm; the first 2 * half elements of every head
+// are rotated, pair (e, e + half) by the angle pos * freq[e], sine and cosine times `magnitude`; v is only converted.
+// Angles are made in double from double frequencies (a token's sines and cosines once, for all its heads); sums of
+// squares and the rotation are 32-bit.  A workgroup per token.
+template <typename T>
+__global__ __launch_bounds__(256) void row_norm_rope_kernel(const float* __restrict__ q, long ldq, const float* __restrict__ k,
+                                                            long ldk, const float* __restrict__ v, long ldv,
+                                                            T* __restrict__ q_out, long ldqo, T* __restrict__ k_out, long ldko,
+                                                            T* __restrict__ v_out, long ldvo, const float* __restrict__ q_w,
+                                                            const float* __restrict__ k_w, float eps_q, float eps_k,
+                                                            const double* __restrict__ freq, int half, float magnitude,
+                                                            const int* __restrict__ tok_pos, int nh, int nkv, int hd, int vd) {
+    __shared__ float cs[2][256];
+    __shared__ float red[16];
+    const int t = blockIdx.x;
+    const int pos = tok_pos[t];
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        const double ang = (double)pos * freq[i];
+        cs[0][i] = (float)(cos(ang) * (double)magnitude);
+        cs[1][i] = (float)(sin(ang) * (double)magnitude);
+    }
+    for (int side = 0; side < 2; ++side) {
+        const float* x = side == 0 ? q + (size_t)t * ldq : (k ? k + (size_t)t * ldk : nullptr);
+        if (!x) continue;                                   // (the whole workgroup: a run that appends nothing has no k)
+        T* y = side == 0 ? q_out + (size_t)t * ldqo : k_out + (size_t)t * ldko;
+        const float* w = side == 0 ? q_w : k_w;
+        const int heads = side == 0 ? nh : nkv, n = heads * hd;
+        float inv = 1.f;
+        if (w) {
+            float sq = 0.f;
+            for (int i = threadIdx.x; i < n; i += blockDim.x) sq = fmaf(x[i], x[i], sq);
+            inv = 1.0f / sqrtf(block_sum(sq, red) / (float)n + (side == 0 ? eps_q : eps_k));
+        } else {
+            __syncthreads();                                // (the table of sines and cosines is complete)
+        }
+        for (int i = threadIdx.x; i < n; i += blockDim.x) {
+            const int e = i % hd;
+            if (e < half) {
+                const float a = x[i] * inv * (w ? w[i] : 1.f), b = x[i + half] * inv * (w ? w[i + half] : 1.f);
+                const float c = cs[0][e], sn = cs[1][e];
+                st(y + i, a * c - b * sn);
+                st(y + i + half, b * c + a * sn);
+            } else if (e >= 2 * half) {
+                st(y + i, x[i] * inv * (w ? w[i] : 1.f));
+            }
+        }
+    }
+    if (v)
+        for (int i = threadIdx.x; i < nkv * vd; i += blockDim.x) st(v_out + (size_t)t * ldvo + i, v[(size_t)t * ldv + i]);
+}
+
+extern "C" int agave_row_norm_rope(int dtype, const float* q, long ldq, const float* k, long ldk, const float* v, long ldv,
+                                   void* q_out, long ldqo, void* k_out, long ldko, void* v_out, long ldvo, const float* q_w,
+                                   const float* k_w, float eps_q, float eps_k, const double* freq, int half, float magnitude,
+                                   const int* tok_pos, int N, int nh, int nkv, int hd, int vd, hipStream_t stream) {
+    AGAVE_CHECK(N >= 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0, "row_norm_rope: bad sizes");
+    AGAVE_CHECK(q && q_out && tok_pos && ldq >= (long)nh * hd && ldqo >= (long)nh * hd, "row_norm_rope: q rows missing or too short");
+    AGAVE_CHECK(!k || (v && k_out && v_out && ldk >= (long)nkv * hd && ldko >= (long)nkv * hd && ldv >= (long)nkv * vd &&
+                       ldvo >= (long)nkv * vd), "row_norm_rope: k and v rows missing or too short");
+    AGAVE_CHECK(half >= 0 && half <= 256 && 2 * half <= hd && (half == 0 || freq), "row_norm_rope: %d rotated pairs in a head of %d (at most 256, with their frequencies)", half, hd);
+    if (N == 0) return 0;
+#define RNR_GO(T_) row_norm_rope_kernel<T_><<<N, 256, 0, stream>>>(q, ldq, k, ldk, k ? v : nullptr, ldv, (T_*)q_out, ldqo, (T_*)k_out, ldko, (T_*)v_out, ldvo, q_w, k_w, eps_q, eps_k, freq, half, magnitude, tok_pos, nh, nkv, hd, vd)
+    if (dtype == AGAVE_F32) RNR_GO(float);
+    else if (dtype == AGAVE_BF16) RNR_GO(bf16);
+    else AGAVE_CHECK(false, "row_norm_rope: unknown dtype %d", dtype);
+#undef RNR_GO
+    AGAVE_LAUNCH_CHECK("row_norm_rope");
+    return 0;
+}
+
 // ------------------------------------------------------------------ what the attention kernels share
 struct BiasedArgs {
     const void* q; long ldq;
@@ -109,6 +184,8 @@ struct BiasedArgs {
     const float* bias; int bias_len;     // slopes [nh], or table [nh][bias_len]
     const float* sink;                   // [nh] or null
     int packed;                          // the pages are in operand order
+    int chunk;                           // 0: none; C: only keys of the query's own chunk of C positions
+    float softcap;                       // 0: none; cap: score <- cap * tanh(score / cap), before the bias
 };
 
 __device__ __forceinline__ float score_bias(const BiasedArgs& A, int h, int dist) {
@@ -134,7 +211,8 @@ __global__ __launch_bounds__(256) void attn_biased_plain_kernel(BiasedArgs A) {
     const int kvh = h / (nh / nkv);
     const int b = A.tok_seq[t];
     const int p = A.tok_pos[t];
-    const int lo = A.window > 0 ? (p - A.window + 1 > 0 ? p - A.window + 1 : 0) : 0;
+    int lo = A.window > 0 ? (p - A.window + 1 > 0 ? p - A.window + 1 : 0) : 0;
+    if (A.chunk > 0) lo = max(lo, (p / A.chunk) * A.chunk);
     const int kept_end = A.keep_first < lo ? A.keep_first : lo;     // keys [0, kept_end) lie before the window
     const int pbase = A.base[b];
     const T* q = (const T*)A.q;
@@ -183,7 +261,9 @@ __global__ __launch_bounds__(256) void attn_biased_plain_kernel(BiasedArgs A) {
                     const T* kr = k_pages + (((size_t)pg * nkv + kvh) * AGAVE_PAGE + (j % AGAVE_PAGE)) * hd;
                     for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], ld(kr + d), dot);
                 }
-                s = dot * A.scale + score_bias(A, h, p - j);
+                s = dot * A.scale;
+                if (A.softcap > 0.f) s = A.softcap * tanhf(s / A.softcap);
+                s += score_bias(A, h, p - j);
             }
             const float cmax = block_max(s, red);
             const float m_new = fmaxf(m, cmax);
@@ -236,6 +316,7 @@ static int check_biased(const BiasedArgs& A, int N) {
     AGAVE_CHECK(A.ldq >= (long)A.nh * A.hd && A.ldo >= (long)A.nh * A.vd && (!A.gate || A.ldg >= (long)A.nh * A.vd),
                 "attn_biased: a row stride is too small");
     AGAVE_CHECK(A.window >= 0 && A.keep_first >= 0 && A.head >= 0, "attn_biased: negative window, kept positions or kept pages");
+    AGAVE_CHECK(A.chunk >= 0 && A.softcap >= 0.f && (A.chunk == 0 || A.keep_first == 0), "attn_biased: a negative chunk or cap, or chunks with kept first positions");
     AGAVE_CHECK(A.keep_first <= A.head * AGAVE_PAGE, "attn_biased: %d kept positions do not fit %d kept pages", A.keep_first, A.head);
     AGAVE_CHECK(A.bias_mode >= 0 && A.bias_mode <= 2 && (A.bias_mode == 0 || A.bias) && (A.bias_mode != 2 || A.bias_len > 0),
                 "attn_biased: bias mode %d without its numbers", A.bias_mode);
@@ -250,9 +331,9 @@ extern "C" int agave_attn_biased_plain(int dtype, const void* q, long ldq, void*
                                        const int* base, int head, int n_pages, const int* tok_seq, const int* tok_pos, int N,
                                        int nh, int nkv, int hd, int vd, float scale, int window, int keep_first,
                                        int bias_mode, const float* bias, int bias_len, const float* sink, int packed,
-                                       hipStream_t stream) {
+                                       int chunk, float softcap, hipStream_t stream) {
     BiasedArgs A{q, ldq, out, ldo, gate, ldg, k_pages, v_pages, table, width, base, head, n_pages, tok_seq, tok_pos,
-                 nh, nkv, hd, vd, scale, window, keep_first, bias_mode, bias, bias_len, sink, packed};
+                 nh, nkv, hd, vd, scale, window, keep_first, bias_mode, bias, bias_len, sink, packed, chunk, softcap};
     AGAVE_CHECK(!packed || dtype == AGAVE_BF16, "attn_biased: pages in operand order hold bfloat16");
     if (check_biased(A, N)) return -1;
     if (N == 0) return 0;
@@ -358,8 +439,14 @@ __global__ __launch_bounds__((KS > 8 || VB > 16) ? 256 : 512) void attn_biased_m
     }
     const int kvh = head / per;
     const int ksl = (hd + 31) / 32;                 // steps along the head that the pages hold
-    const int W = A.window, keep = A.keep_first;
-    const int lo = W > 0 ? max(0, pmin - W + 1) : 0;
+    const int W = A.window, keep = A.keep_first, C = A.chunk;
+    int lo = W > 0 ? max(0, pmin - W + 1) : 0;
+    if (C > 0) lo = max(lo, (pmin / C) * C);           // (the earliest chunk start among the wave's rows)
+    int cstart[NC];                                     // first position of each column's chunk
+#pragma unroll
+    for (int cb = 0; cb < NC; ++cb) cstart[cb] = C > 0 ? (pos[cb] / C) * C : 0;
+    const int cstart_max = C > 0 ? (pmax / C) * C : 0;
+    const float cap2 = A.softcap * 1.4426950408889634f, scale_cap = A.softcap > 0.f ? A.scale / A.softcap : 0.f;
     const int first_win = lo / AGAVE_PAGE;
     const int n_kept = min(first_win, (keep + AGAVE_PAGE - 1) / AGAVE_PAGE);
     const int n_pg = n_kept + pmax / AGAVE_PAGE - first_win + 1;
@@ -527,7 +614,8 @@ __global__ __launch_bounds__((KS > 8 || VB > 16) ? 256 : 512) void attn_biased_m
         frag16 pf[NC][2];
         float alpha[NC];
         const int j_last = pi * AGAVE_PAGE + AGAVE_PAGE - 1;
-        const bool whole = j_last <= pmin && (W == 0 || pmax - pi * AGAVE_PAGE < W || j_last < keep);
+        const bool whole = j_last <= pmin && (W == 0 || pmax - pi * AGAVE_PAGE < W || j_last < keep) &&
+                           (C == 0 || pi * AGAVE_PAGE >= cstart_max);
         auto scores = [&](auto whole_tag, auto table_tag) {
             constexpr bool WHOLE = decltype(whole_tag)::value != 0, TABLE = decltype(table_tag)::value != 0;
 #pragma unroll
@@ -541,9 +629,17 @@ __global__ __launch_bounds__((KS > 8 || VB > 16) ? 256 : 512) void attn_biased_m
                     for (int e = 0; e < 4; ++e) {
                         const int off = 32 * (kb >> 1) + 4 * (kb & 1) + e;  // (a constant once the loops are unrolled)
                         const int dist = d0 - off;
-                        float v = fmaf(s[cb][kb][e], scale2, fmaf(slope2, (float)off, t0));
+                        float v;
+                        if (cap2 > 0.f) {
+                            // cap tanh(x / cap) with tanh(z) = 1 - 2 / (e^(2z) + 1), which is right at both ends
+                            const float e2 = __builtin_amdgcn_exp2f(s[cb][kb][e] * scale_cap * 2.8853900817779268f);
+                            v = fmaf(cap2, 1.0f - 2.0f * __builtin_amdgcn_rcpf(e2 + 1.0f), fmaf(slope2, (float)off, t0));
+                        } else {
+                            v = fmaf(s[cb][kb][e], scale2, fmaf(slope2, (float)off, t0));
+                        }
                         bool see = true;
-                        if (!WHOLE) see = valid[cb] && dist >= 0 && (W == 0 || dist < W || pos[cb] - dist < keep);
+                        if (!WHOLE) see = valid[cb] && dist >= 0 && (W == 0 || dist < W || pos[cb] - dist < keep) &&
+                                          pos[cb] - dist >= cstart[cb];
                         if (TABLE) {
                             int at = dist < A.bias_len ? dist : A.bias_len - 1;
                             if (!WHOLE) at = see ? at : 0;
@@ -652,7 +748,8 @@ __global__ __launch_bounds__((KS > 8 || VB > 16) ? 256 : 512) void attn_biased_m
         const int tbl = M.table_in_lds ? (A.bias_len + 3) / 4 * 4 : 0;         // floats in front of the pages
         lds_u32x4* pages = (lds_u32x4*)(lds + tbl);
         const int n_k = 4 * ksl, n_v = (vd / 16) * 2, buf_tiles = n_k + n_v;
-        const int g_lo = W > 0 ? max(0, wg_first - W + 1) : 0;
+        int g_lo = W > 0 ? max(0, wg_first - W + 1) : 0;
+        if (C > 0) g_lo = max(g_lo, (wg_first / C) * C);
         const int g_first = g_lo / AGAVE_PAGE;
         const int g_kept = min(g_first, (keep + AGAVE_PAGE - 1) / AGAVE_PAGE);
         const int g_n = g_kept + wg_last / AGAVE_PAGE - g_first + 1;
@@ -865,9 +962,10 @@ extern "C" int agave_attn_biased_mfma(const void* q, long ldq, void* out, long l
                                       int head, int n_pages, const int* tok_seq, const int* tok_pos, const int* cu, int N,
                                       int n_seqs, int max_rows, int one_row, int nh, int nkv, int hd, int vd, float scale,
                                       int window, int keep_first, int bias_mode, const float* bias, int bias_len,
-                                      const float* sink, int splits, float* parts, hipStream_t stream) {
+                                      const float* sink, int splits, float* parts, int chunk, float softcap,
+                                      hipStream_t stream) {
     BiasedArgs A{q, ldq, out, ldo, gate, ldg, k_pages, v_pages, table, width, base, head, n_pages, tok_seq, tok_pos,
-                 nh, nkv, hd, vd, scale, window, keep_first, bias_mode, bias, bias_len, sink, 1};
+                 nh, nkv, hd, vd, scale, window, keep_first, bias_mode, bias, bias_len, sink, 1, chunk, softcap};
     if (check_biased(A, N)) return -1;
     AGAVE_CHECK(splits >= 1 && splits <= 64 && (splits == 1 || (one_row && parts)),
                 "attn_biased_mfma: %d shares of a row (1 to 64, in steps of one row a sequence, with memory for them)", splits);

@@ -9,6 +9,9 @@
 //   Expert e < E: W_down[e] (act(W_gate[e] x) * (W_up[e] x)).
 //   The other way of scoring (mode 1): the logits z + bias decide, the `top` largest are chosen, and the weights are
 //   the softmax over the chosen logits alone, times scale.
+//   A third way (mode 2): s = sigmoid(z), each output on its own; choice and groups as with the softmax over all.
+//   `group_top` 2: a group's score is the sum of its two largest c instead of its largest.  `normalise`: the chosen
+//   outputs' weights are divided by their sum + 1e-20 before the factor.
 //   The router matrix may carry further rows behind its R outputs (`extra`): their products with the token are handed
 //   out as they are (the logit of a gate on the shared expert), so that they cost no kernel of their own.
 //
@@ -123,7 +126,7 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
                                                           const float* __restrict__ correction, int N, int K, int R, int groups,
                                                           int keep, int top, float scale, int* __restrict__ choice,
                                                           float* __restrict__ weight, int mode, int extra,
-                                                          float* __restrict__ extra_out) {
+                                                          float* __restrict__ extra_out, int group_top, int normalise) {
     extern __shared__ float zs[];                      // [RR][R + extra], then the corrections [R]
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int Rt = R + extra;
@@ -210,23 +213,39 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
             }
             continue;
         }
-        float mx = -INFINITY;
-        for (int e = lane; e < R; e += 64) mx = fmaxf(mx, sr[e]);
-        mx = wave_max(mx);
-        float sum = 0.f;
-        for (int e = lane; e < R; e += 64) {
-            const float v = expf(sr[e] - mx);
-            sr[e] = v;
-            sum += v;
+        if (mode == 2) {
+            for (int e = lane; e < R; e += 64) sr[e] = 1.0f / (1.0f + expf(-sr[e]));
+        } else {
+            float mx = -INFINITY;
+            for (int e = lane; e < R; e += 64) mx = fmaxf(mx, sr[e]);
+            mx = wave_max(mx);
+            float sum = 0.f;
+            for (int e = lane; e < R; e += 64) {
+                const float v = expf(sr[e] - mx);
+                sr[e] = v;
+                sum += v;
+            }
+            const float inv = 1.0f / wave_sum(sum);
+            for (int e = lane; e < R; e += 64) sr[e] *= inv;
         }
-        const float inv = 1.0f / wave_sum(sum);
-        for (int e = lane; e < R; e += 64) sr[e] *= inv;
+        __builtin_amdgcn_wave_barrier();
         // the groups that stay open: lane g holds group g's score (at most 64 groups)
         unsigned long long open = ~0ull;
         if (keep < groups) {
             float gv = -INFINITY;
-            if (lane < groups)
-                for (int e = lane * gs; e < (lane + 1) * gs; ++e) gv = fmaxf(gv, sr[e] + corr[e]);
+            if (lane < groups) {
+                float second = -INFINITY;
+                for (int e = lane * gs; e < (lane + 1) * gs; ++e) {
+                    const float c = sr[e] + corr[e];
+                    if (c > gv) {
+                        second = gv;
+                        gv = c;
+                    } else {
+                        second = fmaxf(second, c);
+                    }
+                }
+                if (group_top == 2 && gs > 1) gv += second;
+            }
             open = 0ull;
             for (int r = 0; r < keep; ++r) {
                 const float cand = (lane < groups && !((open >> lane) & 1ull)) ? gv : -INFINITY;
@@ -238,7 +257,7 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
         }
         // the `top` best of what is open; what was chosen is marked in the row's sign (s >= 0)
         int my_choice = 0;
-        float my_weight = 0.f;
+        float my_weight = 0.f, chosen_sum = 0.f;
         for (int r = 0; r < top; ++r) {
             float best_v = -INFINITY;
             int best = -1;
@@ -255,6 +274,7 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
             const int chosen = (int)(-wave_max((best >= 0 && best_v == top_v) ? -(float)best : -INFINITY));
             // (top <= open outputs is checked on the host, so some lane has a candidate)
             const float s_chosen = sr[chosen];
+            chosen_sum += s_chosen;
             if ((r & 63) == lane) {             // lane r keeps round r's result; the results leave in one store at the end
                 my_choice = chosen;
                 my_weight = s_chosen * scale;
@@ -266,7 +286,7 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
                 const int at = (r & ~63) + lane;
                 if (at <= r) {
                     choice[(size_t)t * top + at] = my_choice;
-                    weight[(size_t)t * top + at] = my_weight;
+                    weight[(size_t)t * top + at] = normalise ? my_weight / (chosen_sum + 1e-20f) : my_weight;      // (normalise: top <= 64, one batch)
                 }
             }
         }
@@ -275,8 +295,9 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
 
 extern "C" int agave_route_rows(int dtype, const void* x, long ldx, const float* router, const float* correction, int N, int K,
                                 int R, int groups, int keep, int top, float scale, int* choice, float* weight, int mode,
-                                int extra, float* extra_out, hipStream_t stream) {
-    AGAVE_CHECK(mode == 0 || (mode == 1 && top <= 64 && groups == 1), "route_rows: the softmax over the chosen logits takes at most 64 of them and no groups");
+                                int extra, float* extra_out, int group_top, int normalise, hipStream_t stream) {
+    AGAVE_CHECK(mode == 0 || mode == 2 || (mode == 1 && top <= 64 && groups == 1), "route_rows: the softmax over the chosen logits takes at most 64 of them and no groups");
+    AGAVE_CHECK((group_top == 1 || group_top == 2) && (!normalise || (top <= 64 && mode != 1)), "route_rows: a group counts by its largest or its two largest; weights are divided by their sum for at most 64 chosen");
     AGAVE_CHECK(extra >= 0 && extra <= 64 && (extra == 0 || extra_out), "route_rows: %d further rows of the router (0 to 64, with a place for their products)", extra);
     AGAVE_CHECK(N >= 0 && K > 0 && R > 0 && R <= ROUTE_MAX, "route_rows: %d router outputs (1 to %d)", R, ROUTE_MAX);
     AGAVE_CHECK(groups > 0 && groups <= 64 && R % groups == 0, "route_rows: %d outputs in %d groups (equal groups, at most 64)", R, groups);
@@ -289,14 +310,14 @@ extern "C" int agave_route_rows(int dtype, const void* x, long ldx, const float*
     const bool f32 = dtype == AGAVE_F32;
     if (N <= 64) {
         const size_t lds = (size_t)(2 * R + extra) * sizeof(float);
-#define ROUTE_GO(T_, W_) route_rows_kernel<T_, W_, 1><<<N, 1024, lds, stream>>>((const T_*)x, ldx, router, correction, N, K, R, groups, keep, top, scale, choice, weight, mode, extra, extra_out)
+#define ROUTE_GO(T_, W_) route_rows_kernel<T_, W_, 1><<<N, 1024, lds, stream>>>((const T_*)x, ldx, router, correction, N, K, R, groups, keep, top, scale, choice, weight, mode, extra, extra_out, group_top, normalise)
         if (f32 && wide) ROUTE_GO(float, true); else if (f32) ROUTE_GO(float, false); else if (wide) ROUTE_GO(bf16, true); else ROUTE_GO(bf16, false);
 #undef ROUTE_GO
     } else {
         const int blocks = (N + 7) / 8;
         const size_t lds = (size_t)(9 * R + 8 * extra) * sizeof(float);
         const int threads = blocks <= 512 ? 1024 : 256;        // (more waves to share the outputs while they all fit the chip at once)
-#define ROUTE_GO(T_, W_) route_rows_kernel<T_, W_, 8><<<blocks, threads, lds, stream>>>((const T_*)x, ldx, router, correction, N, K, R, groups, keep, top, scale, choice, weight, mode, extra, extra_out)
+#define ROUTE_GO(T_, W_) route_rows_kernel<T_, W_, 8><<<blocks, threads, lds, stream>>>((const T_*)x, ldx, router, correction, N, K, R, groups, keep, top, scale, choice, weight, mode, extra, extra_out, group_top, normalise)
         if (f32 && wide) ROUTE_GO(float, true); else if (f32) ROUTE_GO(float, false); else if (wide) ROUTE_GO(bf16, true); else ROUTE_GO(bf16, false);
 #undef ROUTE_GO
     }

@@ -82,14 +82,19 @@ class Engine:
         # what this element type needs is compiled now, side by side, rather than one library
         # after the other as the first step meets them (a fresh checkout's first run)
         from ..ops import library
-        from ..parts import mixer_libraries
+        from ..parts import lookup, mixer_libraries
         needed = ["elementwise", "gemm"]
         if will_sample:                    # (a caller that only wants logits, like trace replay, builds no sampling kernels)
             needed.append("sampling")
         if self.dtype == torch.bfloat16:
             needed.append("gemm_mfma")
-        for layer in spec.layers:          # what the model's own mixers run on, and no more
+        for layer in spec.layers:          # what the model's own mixers and feed-forwards run on, and no more
             needed += sorted(mixer_libraries(layer.mixer, self.dtype) - set(needed))
+            own = getattr(lookup("ffn", layer.ffn.kind), "kernel_libraries", None) if layer.ffn is not None else None
+            if own is not None:
+                needed += sorted(set(own(layer.ffn, self.dtype)) - set(needed))
+        if spec.streams:
+            needed.append("streams")
         library.ensure_built(needed)
         self.workspace = Workspace(self.device)
         self.env = BuildEnv(self.dtype, self.device, self.workspace, keep_stored_precision=bool(keep_stored_precision))

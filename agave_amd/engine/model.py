@@ -15,7 +15,9 @@ import torch
 from ..cache import GroupKey, StateNeed
 from ..config.spec import ModelSpec
 from ..ops import gemm_mfma, kernels
+from ..ops import streams as stream_ops
 from ..parts import BuildEnv, Linear, add_pending_and_norm, lookup, part_tensors
+from ..parts.streams import write_and_read
 from ..weights.loader import TensorNeed
 
 
@@ -53,6 +55,16 @@ class Model:
             self.head = Linear([self.embed_table], env, "lm_head")      # tied: the same device tensor
             if self.head.packed is not None:
                 self.embed_table = None                                  # rows are gathered from the packed copy
+        # several residual streams: every layer must be of the arrangement that keeps them, and none of the others may be
+        self.streams = int(spec.streams)
+        for layer in spec.layers:
+            if (layer.kind == "streams") != (self.streams > 0):
+                raise ValueError("layers of kind 'streams' and ModelSpec.streams > 0 come together")
+            if self.streams and layer.mixer_streams.streams != self.streams:
+                raise ValueError(f"a layer mixes {layer.mixer_streams.streams} streams, the model has {self.streams}")
+        if self.streams and spec.embed_norm is not None:
+            raise ValueError("several residual streams start as the embedding rows themselves: no norm on them")
+        self.stream_sum = torch.ones(self.streams, dtype=torch.float32, device=env.device) if self.streams else None
         for entry in spec.order:
             if not (0 <= entry.layer < len(self.blocks)):
                 raise ValueError(f"run order names layer {entry.layer}, the model has {len(self.blocks)}")
@@ -99,6 +111,8 @@ class Model:
         """Run the step's tokens through the model; float32 logits [wanted, vocab] or None."""
         ws = self.env.workspace
         n = step.n_tokens
+        if self.streams:
+            return self._forward_streams(step)
         h = ws.get("residual", n, self.spec.hidden, torch.float32)
         pending = None
         rows = h
@@ -120,6 +134,31 @@ class Model:
         # (a decode step wants every row, in order: no gather, and the last branch is added in the norm's kernel)
         rows = None if (step.is_decode and step.n_want == n) else step.want_rows
         add_pending_and_norm(h, pending, self.final_norm, x, rows=rows)   # no final norm: the rows as they are
+        logits = ws.get("logits", step.n_want, self.spec.vocab_size, torch.float32)
+        self.head.forward(x, out=logits)
+        if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0.0:
+            kernels.scale_cap(logits, self.spec.logit_scale, self.spec.logit_softcap)
+        return logits
+
+    def _forward_streams(self, step) -> Optional[torch.Tensor]:
+        """The same with several residual streams a token: they all start as the embedding row, the blocks mix them, and
+        their sum enters the final norm (the last block's result is written by the kernel that sums them)."""
+        ws, n, S, e = self.env.workspace, step.n_tokens, self.streams, self.spec.hidden
+        rows = ws.get("embedded_rows", n, e, torch.float32)
+        if self.embed_table is not None:
+            kernels.embed_scale(step.tokens, self.embed_table, self.spec.embed_scale, rows)
+        else:
+            gemm_mfma.embed_scale_packed(step.tokens, self.head.packed, self.spec.embed_scale, rows, self.spec.vocab_size)
+        h = ws.get("residual_streams", n, S * e, torch.float32)
+        stream_ops.fill(rows, h, S)
+        pending = None
+        for entry in self.spec.order:
+            pending = self.blocks[entry.layer].forward(h, pending, step, entry.memory, entry.writes)
+        if step.n_want == 0:
+            return None
+        x = ws.get("final_normed", step.n_want, e, self.env.dtype)
+        want = None if (step.is_decode and step.n_want == n) else step.want_rows
+        write_and_read(h, S, e, pending, self.stream_sum, self.final_norm, x, rows=want)
         logits = ws.get("logits", step.n_want, self.spec.vocab_size, torch.float32)
         self.head.forward(x, out=logits)
         if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0.0:

@@ -31,10 +31,12 @@ def decode_splits(n_rows: int, n_kv: int, per: int, v_head_dim: int, table_width
 kernels.register_signatures(LIBRARY, {
     "agave_kv_append_rows": [_I, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P],
     "agave_attn_biased_plain": [_I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F,
-                                _I, _I, _I, _P, _I, _P, _I, _P],
+                                _I, _I, _I, _P, _I, _P, _I, _I, _F, _P],
+    "agave_row_norm_rope": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F, _P, _I, _I, _I,
+                            _I, _I, _P],
     "agave_attn_biased_mfma_ok": [_I, _I, _I, _I, _I],
     "agave_attn_biased_mfma": [_P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I,
-                               _F, _I, _I, _I, _P, _I, _P, _I, _P, _P],
+                               _F, _I, _I, _I, _P, _I, _P, _I, _P, _I, _F, _P],
 })
 
 
@@ -84,7 +86,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], 
               v_pages: torch.Tensor, table: torch.Tensor, base: torch.Tensor, head: int, step, n_heads: int, n_kv: int,
               head_dim: int, v_head_dim: int, scale: float, window: Optional[int], keep_first: int, bias_mode: int,
               bias: Optional[torch.Tensor], sink: Optional[torch.Tensor], packed: bool = False,
-              force_plain: bool = False, workspace=None, splits: Optional[int] = None) -> None:
+              force_plain: bool = False, workspace=None, splits: Optional[int] = None, chunk: Optional[int] = None,
+              softcap: float = 0.0) -> None:
     """out[t, h] = sum_j w_j v_j with w = softmax_j(scale q.k_j + bias(h, p - j)) over the keys that token t at
     position p sees (j <= p and (p - j < window or j < keep_first)), the sink's exp(sink_h) added to the
     denominator, times sigmoid(gate[t, h]) element by element.  ``bias``: slopes [heads] (``BIAS_SLOPES``:
@@ -93,7 +96,13 @@ def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], 
     that is a multiple of 16, up to 576 and 512) run on the matrix cores, everything else (and everything with
     ``force_plain``) on the plain kernel, which reads either order.  With a ``workspace`` (something with
     ``get(name, rows, cols, dtype)``) a step of one row a sequence may share a row's pages among several workgroups,
-    whose partial results a second kernel merges (``splits``: how many; None: :func:`decode_splits`)."""
+    whose partial results a second kernel merges (``splits``: how many; None: :func:`decode_splits`).  ``chunk`` C: a
+    token also sees only keys j with j // C == p // C.  ``softcap`` > 0: the scaled score becomes softcap * tanh(score /
+    softcap) before the bias is added."""
+    if chunk is not None and (chunk < 1 or keep_first):
+        raise ValueError("attention: a chunk has at least one position and goes without kept first positions")
+    if softcap < 0:
+        raise ValueError("attention: a cap on the scores is positive (0: none)")
     _dev(q, out, gate, k_pages, v_pages, table, base, bias, sink)
     n = step.n_tokens
     ldq, ldo = _rows(q, "q"), _rows(out, "out")
@@ -136,9 +145,51 @@ def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], 
                      ptr(table), width, ptr(base), head, n_pages, ptr(step.tok_seq), ptr(step.tok_pos), ptr(step.cu_dev), n,
                      step.n_seqs, max_rows, one_row, n_heads, n_kv, head_dim, v_head_dim, float(scale), int(window or 0),
                      int(keep_first), bias_mode, ptr(bias) if bias_mode != BIAS_NONE else None, bias_len, ptr(sink), splits,
-                     ptr(parts), stream())
+                     ptr(parts), int(chunk or 0), float(softcap), stream())
         return
     library.call(_lib(), "agave_attn_biased_plain", dt(q), ptr(q), ldq, ptr(out), ldo, ptr(gate), ldg, ptr(k_pages),
                  ptr(v_pages), ptr(table), width, ptr(base), head, n_pages, ptr(step.tok_seq), ptr(step.tok_pos), n,
                  n_heads, n_kv, head_dim, v_head_dim, float(scale), int(window or 0), int(keep_first), bias_mode,
-                 ptr(bias) if bias_mode != BIAS_NONE else None, bias_len, ptr(sink), 1 if packed else 0, stream())
+                 ptr(bias) if bias_mode != BIAS_NONE else None, bias_len, ptr(sink), 1 if packed else 0, int(chunk or 0),
+                 float(softcap), stream())
+
+
+def row_norm_rope(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], q_out: torch.Tensor,
+                  k_out: Optional[torch.Tensor], v_out: Optional[torch.Tensor], q_weight: Optional[torch.Tensor],
+                  k_weight: Optional[torch.Tensor], eps_q: float, eps_k: float, freq: Optional[torch.Tensor],
+                  magnitude: float, step, n_heads: int, n_kv: int, head_dim: int, v_head_dim: int) -> None:
+    """The 32-bit rows of a step's q, k and v (column slices are fine) into the rows the attention reads and the cache
+    holds, in ``q_out``'s element type: q and k divided by the root mean square of their whole row and multiplied by a
+    weight per element (where a weight is given), then each head's first ``2 * len(freq)`` elements rotated, pair
+    (e, e + len(freq)) by the angle ``pos * freq[e]`` (float64 frequencies), sine and cosine times ``magnitude``; v
+    converted.  ``k`` None: only q (a run that appends nothing)."""
+    _dev(q, k, v, q_out, k_out, v_out, q_weight, k_weight, freq)
+    n = step.n_tokens
+
+    def f32rows(t, what, cols):
+        if t.dtype != torch.float32 or t.dim() != 2 or t.stride(1) != 1 or tuple(t.shape) != (n, cols):
+            raise ValueError(f"row_norm_rope: {what} must be float32 rows [{n}, {cols}], got {tuple(t.shape)} {t.dtype}")
+        return t.stride(0)
+
+    def outrows(t, what, cols):
+        if t.dtype != q_out.dtype or t.dim() != 2 or t.stride(1) != 1 or tuple(t.shape) != (n, cols):
+            raise ValueError(f"row_norm_rope: {what} must be rows [{n}, {cols}] of the result's dtype")
+        return t.stride(0)
+    qd, kd, vd = n_heads * head_dim, n_kv * head_dim, n_kv * v_head_dim
+    ldq, ldqo = f32rows(q, "q", qd), outrows(q_out, "q_out", qd)
+    ldk = ldv = ldko = ldvo = 0
+    if k is not None:
+        ldk, ldv = f32rows(k, "k", kd), f32rows(v, "v", vd)
+        ldko, ldvo = outrows(k_out, "k_out", kd), outrows(v_out, "v_out", vd)
+    _f32vec(q_weight, "q weight", qd)
+    _f32vec(k_weight, "k weight", kd)
+    half = 0
+    if freq is not None:
+        if freq.dtype != torch.float64 or not freq.is_contiguous():
+            raise TypeError("row_norm_rope: frequencies are a contiguous float64 vector")
+        half = freq.numel()
+        if 2 * half > head_dim or half > 256:
+            raise ValueError(f"row_norm_rope: {2 * half} rotated elements in a head of {head_dim} (at most 512)")
+    library.call(_lib(), "agave_row_norm_rope", dt(q_out), ptr(q), ldq, ptr(k), ldk, ptr(v), ldv, ptr(q_out), ldqo, ptr(k_out),
+                 ldko, ptr(v_out), ldvo, ptr(q_weight), ptr(k_weight), float(eps_q), float(eps_k), ptr(freq), half,
+                 float(magnitude), ptr(step.tok_pos), n, n_heads, n_kv, head_dim, v_head_dim, stream())

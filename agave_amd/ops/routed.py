@@ -14,7 +14,7 @@ MAX_OUTPUTS = 1024
 kernels.register_signatures(LIBRARY, {
     "agave_route_topk": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _F, _P, _P, _P],
     "agave_routed_experts_plain": [_I, _P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _F, _P],
-    "agave_route_rows": [_I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P, _I, _I, _P, _P],
+    "agave_route_rows": [_I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P, _I, _I, _P, _I, _I, _P],
     "agave_route_sort": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
     "agave_routed_experts_mfma": [_P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
     "agave_routed_combine": [_I, _P, _P, _P, _P, _P, _L, _P, _L, _P, _P, _L, _I, _I, _I, _I, _P],
@@ -150,13 +150,16 @@ def experts_mfma(x: torch.Tensor, sorted_pair: torch.Tensor, tile_expert: torch.
 
 def route_rows(x: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int, top: int,
                scale: float, choice: torch.Tensor, weight: torch.Tensor, softmax_top: bool = False,
-               extra_out: Optional[torch.Tensor] = None) -> None:
+               extra_out: Optional[torch.Tensor] = None, sigmoid: bool = False, group_top: int = 1,
+               normalise: bool = False) -> None:
     """The router's 32-bit product ``x router^T`` and :func:`route_topk`'s choice in one kernel (the logits never
     leave the compute unit).  ``router`` is float32 [R, width]; ``x`` [N, width] in either element type.
     ``softmax_top``: the ``top`` largest logits + ``correction`` are chosen (the lower index among equals) and their
     weights are the softmax over the chosen alone, times ``scale`` (no groups, ``top`` <= 64).  ``extra_out``
     (float32 [N, extra]): the router matrix has ``extra`` further rows behind its outputs, whose products with
-    the rows are left there as they are."""
+    the rows are left there as they are.  ``sigmoid``: the scores are the logits' sigmoids instead of their softmax.
+    ``group_top`` 2: a group counts by the sum of its two largest scores + correction.  ``normalise``: the chosen
+    weights are divided by their sum + 1e-20 before ``scale`` (``top`` <= 64)."""
     _dev(x, router, correction, choice, weight, extra_out)
     n, k = x.shape
     ldx = _rows(x, "x")
@@ -172,12 +175,18 @@ def route_rows(x: torch.Tensor, router: torch.Tensor, correction: Optional[torch
         raise ValueError("route_rows: the router has no outputs")
     if softmax_top and (groups != 1 or keep != 1 or top > 64):
         raise ValueError("route_rows: the softmax over the chosen logits takes no groups and at most 64 chosen")
+    if softmax_top and (sigmoid or normalise):
+        raise ValueError("route_rows: one way of scoring at a time")
+    if group_top not in (1, 2) or (normalise and top > 64):
+        raise ValueError("route_rows: a group counts by its largest or its two largest scores; weights are divided by their "
+                         "sum for at most 64 chosen")
     _f32vec(correction, "correction", r)
     _i32(choice, "choice", n * top)
     if weight.dtype != torch.float32 or not weight.is_contiguous() or weight.numel() < n * top:
         raise ValueError("route_rows: weight must be contiguous float32 [N, top]")
     library.call(_lib(), "agave_route_rows", dt(x), ptr(x), ldx, ptr(router), ptr(correction), n, k, r, groups, keep, top,
-                 float(scale), ptr(choice), ptr(weight), 1 if softmax_top else 0, extra, ptr(extra_out), stream())
+                 float(scale), ptr(choice), ptr(weight), 1 if softmax_top else (2 if sigmoid else 0), extra, ptr(extra_out),
+                 int(group_top), 1 if normalise else 0, stream())
 
 
 def pack_expert_weights(w: torch.Tensor) -> torch.Tensor:

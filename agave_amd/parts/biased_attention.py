@@ -14,6 +14,11 @@ from which the last bucket holds), so the kernels know a slope or a table and no
 A mixer without key and value projections appends nothing and reads the memory that its run-order
 entry names (another layer's keys and values as the cache holds them), through its own mask.
 
+A mixer may besides have biases on its q, k and v products, an RMS norm over the whole row of q and of k (all heads
+side by side) followed by a rotation of each head's first elements, a cap on the scaled scores, and chunks of
+positions instead of (or besides) a window.  With a norm or a rotation the first product leaves 32-bit rows, and one
+kernel norms, rotates and rounds them to the engine's element type once.
+
 Scores, bias, softmax and the sums over the values are 32-bit in both engines.
 """
 from __future__ import annotations
@@ -26,8 +31,9 @@ import torch
 from ..cache import GroupKey, StateNeed
 from ..config.spec import BiasedAttentionSpec, ScoreBiasSpec
 from ..ops import attention_biased as ops
+from ..ops import kernels
 from ..weights.loader import TensorNeed
-from .base import BuildEnv, register
+from .base import BuildEnv, lookup, register
 from .linear import Linear
 
 
@@ -74,16 +80,47 @@ class BiasedAttention:
         self.qd, self.kd, self.vd = s.n_heads * s.head_dim, s.n_kv_heads * s.head_dim, s.n_kv_heads * s.v_head_dim
         self.ctx = s.n_heads * s.v_head_dim
         self.own_kv = bool(s.k_proj)
-        mats = [weights.get(s.q_proj)]
+        def bias(name):
+            return weights.get(name) if name else None
+        mats, biases = [weights.get(s.q_proj)], [bias(s.q_bias)]
         bounds = [0, self.qd]
         if self.own_kv:
             mats += [weights.get(s.k_proj), weights.get(s.v_proj)]
+            biases += [bias(s.k_bias), bias(s.v_bias)]
             bounds += [bounds[-1] + self.kd, bounds[-1] + self.kd + self.vd]
+        elif s.k_bias or s.v_bias or s.k_row_norm is not None:
+            raise ValueError("biased attention: a mixer without key and value projections has no biases or norm for them")
         if s.gate_proj:
             mats.append(weights.get(s.gate_proj))
+            biases.append(None)
             bounds.append(bounds[-1] + self.ctx)
         self._bounds = tuple(bounds)
-        self.proj = Linear(mats, env, "qkvg")          # one product for everything that reads the mixer's input
+        self.proj = Linear(mats, env, "qkvg", biases=biases)    # one product for everything that reads the mixer's input
+        # the norm over whole rows and the rotation: q and k pass a kernel of their own on their way
+        self.q_weight = self.k_weight = None
+        self.q_eps = self.k_eps = 0.0
+        for which, ns, size in (("q", s.q_row_norm, self.qd), ("k", s.k_row_norm, self.kd)):
+            if ns is None:
+                continue
+            if ns.kind != "rmsnorm" or ns.size != size or ns.bias:
+                raise ValueError(f"biased attention: the norm over the {which} rows must be an RMS norm of {size} elements")
+            w = weights.get(ns.weight).to(torch.float32)
+            w = (w + 1.0 if ns.add_one else w).contiguous().to(env.device)
+            if which == "q":
+                self.q_weight, self.q_eps = w, float(ns.eps)
+            else:
+                self.k_weight, self.k_eps = w, float(ns.eps)
+        self.position = lookup("position", s.position.kind)(s.position, env)
+        table = getattr(self.position, "rotation_table", None)
+        if table is None:
+            raise ValueError(f"biased attention: the position encoding {s.position.kind!r} is no rotation of pairs")
+        self.freq, interleaved = table()
+        if interleaved:
+            raise ValueError("biased attention: rotated pairs are (e, e + rotary_dim / 2)")
+        self.magnitude = float(getattr(self.position, "magnitude", 1.0))
+        self.prepares_rows = self.q_weight is not None or self.k_weight is not None or self.freq is not None
+        if s.chunk is not None and s.keep_first:
+            raise ValueError("biased attention: chunks go without kept first positions")
         self.o = Linear([weights.get(s.o_proj)], env, "attn_o")
         self.sink = weights.get(s.sink).to(torch.float32).contiguous().to(env.device) if s.sink else None
         b = s.bias
@@ -112,11 +149,17 @@ class BiasedAttention:
         if s.gate_proj:
             needs.append(TensorNeed(s.gate_proj, (ctx, s.hidden)))
         needs.append(TensorNeed(s.o_proj, (s.hidden, ctx)))
+        for name, size in ((s.q_bias, qd), (s.k_bias, kd), (s.v_bias, vd)):
+            if name:
+                needs.append(TensorNeed(name, (size,)))
+        for ns in (s.q_row_norm, s.k_row_norm):
+            if ns is not None:
+                needs.append(TensorNeed(ns.weight, (ns.size,)))
         return needs
 
     def kv_need(self) -> Optional[GroupKey]:
         s = self.spec
-        return GroupKey(s.window, s.n_kv_heads, s.head_dim, v_head_dim=s.v_head_dim, layout="rows_vt",
+        return GroupKey(s.window, s.n_kv_heads, s.head_dim, chunk=s.chunk, v_head_dim=s.v_head_dim, layout="rows_vt",
                         keep_first=s.keep_first if s.window is not None else 0)
 
     def state_need(self) -> Optional[StateNeed]:
@@ -132,18 +175,36 @@ class BiasedAttention:
         k_pages, v_pages, packed = step.cache.pages_of(memory)
         table, base = step.tables[group]
         head = step.cache.group_keys[group].kept_pages
-        proj = self.proj.forward(x, tag="qkvg")
-        cols = ws.columns(proj, self._bounds)
-        q = cols[0]
-        at = 1
+        if self.prepares_rows:
+            # 32-bit rows from the product; norm, rotation and the one rounding to the engine's type in one kernel
+            proj = self.proj.forward(x, out_dtype=torch.float32, tag="qkvg32")
+            cols = ws.columns(proj, self._bounds)
+            q = ws.get("attn_q_rows", n, self.qd, x.dtype)
+            k = v = None
+            if self.own_kv:
+                kv = ws.get("attn_kv_rows", n, self.kd + self.vd, x.dtype)
+                k, v = ws.columns(kv, (0, self.kd, self.kd + self.vd))
+            ops.row_norm_rope(cols[0], cols[1] if self.own_kv else None, cols[2] if self.own_kv else None, q, k, v,
+                              self.q_weight, self.k_weight, self.q_eps, self.k_eps, self.freq, self.magnitude, step,
+                              s.n_heads, s.n_kv_heads, s.head_dim, s.v_head_dim)
+            gate = None
+            if s.gate_proj:
+                g32 = cols[3 if self.own_kv else 1]
+                gate = ws.get("attn_gate_rows", n, self.ctx, x.dtype)
+                kernels.cast(g32, gate)
+        else:
+            proj = self.proj.forward(x, tag="qkvg")
+            cols = ws.columns(proj, self._bounds)
+            q = cols[0]
+            k, v = (cols[1], cols[2]) if self.own_kv else (None, None)
+            gate = cols[3 if self.own_kv else 1] if s.gate_proj else None
         if self.own_kv:
-            ops.kv_append_rows(cols[1], cols[2], k_pages, v_pages, table, base, head, step, s.n_kv_heads, s.head_dim,
+            ops.kv_append_rows(k, v, k_pages, v_pages, table, base, head, step, s.n_kv_heads, s.head_dim,
                                s.v_head_dim, packed)
-            at = 3
-        gate = cols[at] if s.gate_proj else None
         ctx = ws.get("attn_ctx", n, self.ctx, x.dtype)
         ops.attention(q, ctx, gate, k_pages, v_pages, table, base, head, step, s.n_heads, s.n_kv_heads, s.head_dim,
-                      s.v_head_dim, s.scale, s.window, s.keep_first, self.bias_mode, self.bias, self.sink, packed)
+                      s.v_head_dim, s.scale, s.window, s.keep_first, self.bias_mode, self.bias, self.sink, packed,
+                      workspace=ws, chunk=s.chunk, softcap=s.softcap)
         return self.o.forward(ctx, tag="attn_o", slices_ok=True)       # the block adds it to the residual stream
 
 

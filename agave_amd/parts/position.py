@@ -8,6 +8,7 @@ in 32-bit inside the q/k kernel.  ``none``: nothing is applied.
 """
 from __future__ import annotations
 
+import math
 from typing import Optional, Tuple
 
 import numpy as np
@@ -30,6 +31,7 @@ class RotaryPosition:
         self.rotary_dim = spec.rotary_dim
         self.interleaved = bool(spec.interleaved)
         self._exact = inv / float(spec.factor)
+        self.magnitude = 1.0           # a factor on sine and cosine (1: a pure rotation)
         self._freq64: Optional[torch.Tensor] = None
         self._device = env.device
 
@@ -44,6 +46,33 @@ class RotaryPosition:
         return self._freq64, self.interleaved
 
 
+class YarnRotaryPosition(RotaryPosition):
+    """The same rotation with YaRN's frequencies: pair i's frequency ``f_i = theta^(-2i/d)`` becomes
+    ``f_i / s * r_i + f_i (1 - r_i)`` for the factor s, with ``r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)``,
+    ``lo = max(floor(w(fast)), 0)``, ``hi = min(ceil(w(slow)), d - 1)`` and ``w(t) = d ln(original / (2 pi t)) / (2 ln theta)``:
+    pairs that turn often within the original context keep their frequency, pairs that turn less than once are slowed
+    down by s, those between are blended.  Sine and cosine are multiplied by ``magnitude = slope ln(s) + 1``.  The
+    frequencies are made in double; a kernel that makes the angle in double reads them through ``rotation_table``."""
+
+    def __init__(self, spec: PositionSpec, env: BuildEnv):
+        super().__init__(PositionSpec("rope", rotary_dim=spec.rotary_dim, theta=spec.theta, interleaved=spec.interleaved), env)
+        if spec.yarn_factor <= 0 or spec.yarn_original < 1 or spec.yarn_fast <= 0 or spec.yarn_slow <= 0 or spec.theta == 1.0:
+            raise ValueError("rope_yarn needs a positive factor, original context, fast and slow turn counts, and theta != 1")
+        d = spec.rotary_dim
+
+        def where(turns: float) -> float:
+            return d * math.log(spec.yarn_original / (2.0 * math.pi * turns)) / (2.0 * math.log(spec.theta))
+        lo, hi = max(math.floor(where(spec.yarn_fast)), 0), min(math.ceil(where(spec.yarn_slow)), d - 1)
+        i = np.arange(d // 2, dtype=np.float64)
+        ramp = np.clip((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        self._exact = self._exact / float(spec.yarn_factor) * ramp + self._exact * (1.0 - ramp)
+        self.inv_freq = torch.from_numpy(self._exact.astype(np.float32)).to(env.device)
+        self.magnitude = float(spec.yarn_magnitude_slope * math.log(spec.yarn_factor) + 1.0)
+
+    def fused_rotation(self):
+        raise ValueError("rope_yarn scales sine and cosine: the q/k kernel of the plain rotation does not apply it")
+
+
 class NoPosition:
     def __init__(self, spec: PositionSpec, env: BuildEnv):
         pass
@@ -56,4 +85,5 @@ class NoPosition:
 
 
 register("position", "rope", RotaryPosition)
+register("position", "rope_yarn", YarnRotaryPosition)
 register("position", "none", NoPosition)

@@ -43,8 +43,11 @@ class RoutedFfn:
             raise ValueError(f"routed feed-forward: {s.keep_groups} of {s.groups} groups kept")
         if not 1 <= s.top <= s.keep_groups * (self.n_outputs // s.groups):
             raise ValueError(f"routed feed-forward: {s.top} experts chosen of {s.keep_groups * (self.n_outputs // s.groups)} that can be")
-        if s.score not in ("softmax_all", "softmax_top"):
-            raise ValueError(f"routed feed-forward: unknown way of scoring {s.score!r} (softmax_all, softmax_top)")
+        if s.score not in ("softmax_all", "softmax_top", "sigmoid"):
+            raise ValueError(f"routed feed-forward: unknown way of scoring {s.score!r} (softmax_all, softmax_top, sigmoid)")
+        if s.group_top not in (1, 2) or (s.normalise and (s.top > 64 or s.score == "softmax_top")):
+            raise ValueError("routed feed-forward: a group counts by its largest or its two largest scores; weights are divided "
+                             "by their sum for at most 64 chosen experts")
         if s.score == "softmax_top" and (s.groups != 1 or s.top > 64 or s.n_identity):
             raise ValueError("routed feed-forward: the softmax over the chosen logits takes no groups, no identity experts "
                              "and at most 64 chosen")
@@ -99,7 +102,8 @@ class RoutedFfn:
         # the router's 32-bit product and the choice in one kernel
         shared_gate = ws.get("router_shared_gate", n, 1, torch.float32) if s.shared_gate else None
         routed.route_rows(x, self.router, self.correction, s.groups, s.keep_groups, top, s.route_scale, choice, weight,
-                          softmax_top=s.score == "softmax_top", extra_out=shared_gate)
+                          softmax_top=s.score == "softmax_top", extra_out=shared_gate, sigmoid=s.score == "sigmoid",
+                          group_top=s.group_top, normalise=s.normalise)
         y = place = None
         if self.tile_order and not routed.mfma_ok(x, s.intermediate):
             raise ValueError("routed feed-forward: its experts are kept in tile order, which takes aligned bfloat16 rows")
