@@ -14,8 +14,8 @@
 #include "common_impl.h"
 #include <math.h>
 
-#define STREAMS_MAX 8
-#define STREAMS_MAX_WIDTH 16384
+#define STREAMS_MAX 16
+#define STREAMS_MAX_WIDTH 15360
 
 struct StreamsArgs {
     float* h; int S; int E;

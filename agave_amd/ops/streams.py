@@ -9,7 +9,7 @@ from . import kernels, library
 from .kernels import _P, _I, _L, _F, _dev, _f32vec, _i32, dt, ptr, stream
 
 LIBRARY = "streams"
-MAX_STREAMS, MAX_WIDTH = 8, 16384
+MAX_STREAMS, MAX_WIDTH = 16, 15360
 NORM_NONE, NORM_LAYER, NORM_RMS = 0, 1, 2
 
 kernels.register_signatures(LIBRARY, {

@@ -39,7 +39,8 @@ class StreamMix:
     @staticmethod
     def tensor_needs(spec: StreamMixSpec) -> List[TensorNeed]:
         s = spec.streams
-        return [TensorNeed(spec.read, (s,)), TensorNeed(spec.write, (s,)), TensorNeed(spec.mix, (s, s))]
+        return [TensorNeed(spec.read, (s,), init="mean"), TensorNeed(spec.write, (s,), init="ones"),
+                TensorNeed(spec.mix, (s, s), init="identity")]
 
 
 def _norm_arguments(norm):

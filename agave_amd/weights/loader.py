@@ -37,6 +37,9 @@ class TensorNeed:
     name: str
     shape: Tuple[int, ...]
     kind: str = "float"         # "float": a matrix or vector of floats; "int": an integer table
+    # what random weights look like where zero-mean noise would make the model degenerate: "": noise; "identity": the
+    # identity matrix plus noise; "ones": 1 plus noise; "mean": 1/n plus noise (a vector that averages n things)
+    init: str = ""
 
     def accepts(self, stored: str) -> bool:
         return stored in (FLOAT_STORAGE if self.kind == "float" else INT_STORAGE)

@@ -25,8 +25,20 @@ def random_tensors(needs, seed: int, dtype: torch.dtype = torch.bfloat16,
     for i, need in enumerate(needs):
         g = torch.Generator().manual_seed((int(seed) * 1_000_003 + i) & 0x7FFFFFFFFFFFFFFF)
         s = norm_std if len(need.shape) == 1 else std
-        out[need.name] = (torch.randn(need.shape, generator=g, dtype=torch.float32) * s).to(dtype)
+        out[need.name] = (torch.randn(need.shape, generator=g, dtype=torch.float32) * s + _centre(need, torch.device("cpu"))).to(dtype)
     return out
+
+
+def _centre(need, device):
+    """What the noise of a random tensor is added to (``TensorNeed.init``)."""
+    init = getattr(need, "init", "")
+    if init == "identity":
+        return torch.eye(need.shape[0], need.shape[1], dtype=torch.float32, device=device)
+    if init == "ones":
+        return 1.0
+    if init == "mean":
+        return 1.0 / max(int(need.shape[0]), 1)
+    return 0.0
 
 
 def write_random_model(raw_config: dict, seed: int, out_dir: str,
@@ -61,4 +73,7 @@ class RandomWeightSource:
         s = self._norm_std if len(need.shape) == 1 else self._std
         t = torch.empty(need.shape, dtype=torch.float32 if len(need.shape) == 1 else self._dtype, device=self._device)
         t.normal_(0.0, s, generator=g)
+        centre = _centre(need, self._device)
+        if not isinstance(centre, float) or centre != 0.0:
+            t += centre
         return t

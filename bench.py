@@ -23,7 +23,7 @@ The other published shapes:
 
 Another design beside the closest Gemma 3 shape of equal size (not the default run):
 
-    python bench.py --design rilenex|gusedra|batasun [--design-size small|medium|large] [--design-layers 8]
+    python bench.py --design rilenex|gusedra|batasun|duperax [--design-size small|medium|large] [--design-layers 8]
 
 prints one JSON line with, for that decoder and for a Gemma 3 decoder of the same width, depth,
 heads and about as many weights: tokens a second of a 2,048-token prompt and of decode steps at
@@ -269,6 +269,28 @@ def batasun_config(size: str, layers: int) -> dict:
     return {"architecture": "Batasun", "vocab": 32768, "width": e, "norm": {"eps": 1e-5}, "layers": out}
 
 
+def duperax_config(size: str, layers: int) -> dict:
+    """Of every four layers the first has windowed attention whose q and k rows are normed whole, the third attention in
+    chunks with biases, a YaRN rotation and capped scores, the second and fourth the gated linear recurrence (as wide
+    as the model, gates in blocks of 128 channels, four taps); feed-forwards in turn dense (clamped swish) and routed
+    (16 experts of a quarter of the dense inner size in 4 groups of which 2 are open, 4 experts a token, sigmoid
+    scores): a token's routed layer computes as much as a dense one of two thirds the size.  Four residual streams.
+    Heads of 128, a window and chunks of 1,024 positions as the Gemma 3 shape beside it."""
+    e, ff, h, g, d, _, _ = DESIGN_SIZES[size]
+    dense = {"kind": "dense", "ff": (2 * ff // 3) // 256 * 256, "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 16, "top": 4, "groups": {"count": 4, "keep": 2}}}
+    first = {"type": "attention", "mixer": {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 1024}}}
+    second = {"type": "attention_2",
+              "mixer": {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 1024}, "softcap": 30.0,
+                        "rot": {"dims": d, "base": 10000.0, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    lru = {"type": "rglru", "mixer": {"width": e, "blocks": e // 128, "conv": 4}}
+    out = []
+    for i in range(layers):
+        out.append(dict((first, lru, second, lru)[i % 4], mlp=moe if i % 2 else dense))
+    return {"architecture": "Duperax", "vocab": 32768, "width": e, "norm": {"eps": 1e-5}, "streams": 4, "logit_scale": 1.0,
+            "layers": out}
+
+
 def gemma_like_config(size: str, layers: int) -> dict:
     """The same width, depth and heads as a Gemma 3 decoder; its gated feed-forward has three matrices,
     so two thirds of the inner size give as many weights."""
@@ -317,10 +339,12 @@ def compare_designs(args) -> int:
     result = {"metric": f"{args.design} beside Gemma 3 at equal size ({size}, {layers} layers): tokens/s", "unit": "tokens/s",
               "dtype": "bf16", "data": "synthetic: uniform-random token ids, random weights", "sizes": DESIGN_SIZES[size],
               "peaks_measured": measured_peaks()}
-    makers = {"rilenex": rilenex_config, "gusedra": gusedra_config, "batasun": batasun_config}
+    makers = {"rilenex": rilenex_config, "gusedra": gusedra_config, "batasun": batasun_config, "duperax": duperax_config}
     runs = [(args.design, makers[args.design](size, layers))]
-    if args.design == "batasun":          # the design with routed feed-forwards and shared keys stands beside it too
+    if args.design in ("batasun", "duperax"):      # the design with the same attention kernels and routed feed-forwards stands beside it too
         runs.append(("gusedra_equal_size", gusedra_config(size, layers)))
+    if args.design == "duperax":                   # and the one with recurrent layers
+        runs.append(("rilenex_equal_size", rilenex_config(size, layers)))
     runs.append(("gemma3_equal_size", gemma_like_config(size, layers)))
     for name, cfg in runs:
         engine = Engine.from_random(cfg, seed=0, dtype="bfloat16", max_slots=batch, max_context=context,
@@ -361,7 +385,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="time only the 2048-token prefill and print its record (for profiles)")
-    ap.add_argument("--design", choices=["rilenex", "gusedra", "batasun"], help="measure this design beside a Gemma 3 decoder of equal size")
+    ap.add_argument("--design", choices=["rilenex", "gusedra", "batasun", "duperax"], help="measure this design beside a Gemma 3 decoder of equal size")
     ap.add_argument("--design-size", default="medium", choices=sorted(DESIGN_SIZES))
     ap.add_argument("--design-layers", type=int, default=8)
     args = ap.parse_args()

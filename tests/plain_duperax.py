@@ -103,9 +103,10 @@ def tensor_shapes(cfg: dict) -> Dict[str, tuple]:
     return out
 
 
-def random_weights(cfg: dict, seed: int, matrix_std: Optional[float] = None) -> Dict[str, torch.Tensor]:
+def random_weights(cfg: dict, seed: int, matrix_std: Optional[float] = None, decided_routing: bool = False) -> Dict[str, torch.Tensor]:
     """Weights that keep activations of order one through many layers, rounded to bfloat16 values (so that a
-    bfloat16 checkpoint holds exactly these numbers)."""
+    bfloat16 checkpoint holds exactly these numbers).  ``decided_routing``: the corrections of the routers lie two
+    apart, so that no rounding of a score changes which experts are chosen."""
     g = torch.Generator().manual_seed(seed)
     out = {}
     for name, shape in tensor_shapes(cfg).items():
@@ -124,6 +125,8 @@ def random_weights(cfg: dict, seed: int, matrix_std: Optional[float] = None) -> 
             t = torch.randn(shape, generator=g, dtype=F) - 1.0
         elif last == "correction":
             t = 0.2 * torch.randn(shape, generator=g, dtype=F)
+            if decided_routing:
+                t = 2.0 * torch.randperm(shape[0], generator=g).to(F)
         elif last == "conv":
             t = 0.5 * torch.randn(shape, generator=g, dtype=F)
         elif name == "embed":
@@ -149,6 +152,16 @@ def row_rms(x, w, eps):
 
 def gelu_tanh(z):
     return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+
+
+def streams_read(xs, read):
+    """u = sum_s read[s] x_s for streams xs [S, T, E]."""
+    return torch.einsum("s,ste->te", read, xs)
+
+
+def streams_write(xs, y, mix, write):
+    """x_t <- sum_s mix[s, t] x_s + write[t] y, all t at once."""
+    return torch.einsum("st,sne->tne", mix, xs) + write[:, None, None] * y[None]
 
 
 def run_order(cfg: dict) -> List[int]:
@@ -206,16 +219,24 @@ def attention(h, w, p, m, kind, eps):
     if kind == "attention_2":
         pos = torch.arange(T)
         q, k = rotate(q, pos, m["rot"]), rotate(k, pos, m["rot"])
-    see = visible(kind, m["mask"]["size"], T)
-    out = torch.zeros(T, H, dv, dtype=F)
+    see = visible(kind, m["mask"]["size"], T) if m.get("mask") else visible("attention", T, T)
+    cap = m.get("softcap") if kind == "attention_2" else None
+    return softmax_attention(q, k, v, m["scale"], see, cap).reshape(T, H * dv) @ w[p + "o"].T
+
+
+def softmax_attention(q, k, v, scale, see, softcap=None):
+    """q [T, H, d], k [T, G, d], v [T, G, dv]; head h reads key head h // (H / G); ``see`` [T, T] says which keys a
+    query sees.  Returns [T, H, dv]."""
+    T, H, G = q.shape[0], q.shape[1], k.shape[1]
+    out = torch.zeros(T, H, v.shape[2], dtype=F)
     for hh in range(H):
         g = hh // (H // G)
-        s = (q[:, hh] @ k[:, g].T) * m["scale"]
-        if kind == "attention_2" and m.get("softcap"):
-            s = m["softcap"] * torch.tanh(s / m["softcap"])
+        s = (q[:, hh] @ k[:, g].T) * scale
+        if softcap:
+            s = softcap * torch.tanh(s / softcap)
         s = s.masked_fill(~see, -math.inf)
         out[:, hh] = torch.softmax(s, -1) @ v[:, g]
-    return out.reshape(T, H * dv) @ w[p + "o"].T
+    return out
 
 
 def causal_conv(x, taps_w, bias):
@@ -228,21 +249,31 @@ def causal_conv(x, taps_w, bias):
     return out + bias
 
 
+def rglru_gates(u, w_r, b_r, w_i, b_i, lam, c=8.0):
+    """(a, gated input) from the convolved branch u [T, W]; the gate matrices are [blocks, out, in]."""
+    T, nb = u.shape[0], w_r.shape[0]
+    ub = u.view(T, nb, -1)
+    r = torch.sigmoid(torch.einsum("tbi,boi->tbo", ub, w_r) + b_r).reshape(T, -1)
+    g = torch.sigmoid(torch.einsum("tbi,boi->tbo", ub, w_i) + b_i).reshape(T, -1)
+    a = torch.exp(-c * r * torch.nn.functional.softplus(lam))
+    return a, torch.sqrt(1.0 - a ** 2) * g * u
+
+
+def linear_scan(a, x):
+    """S_t = a_t S_(t-1) + x_t from S = 0; all S_t [T, W]."""
+    S = torch.zeros(a.shape[1], dtype=F)
+    out = torch.zeros_like(x)
+    for t in range(a.shape[0]):
+        S = a[t] * S + x[t]
+        out[t] = S
+    return out
+
+
 def rglru(h, w, p, m):
-    T, nb = h.shape[0], m["blocks"]
     y = gelu_tanh(h @ w[p + "y"].T + w[p + "y.b"])
     u = causal_conv(h @ w[p + "x"].T + w[p + "x.b"], w[p + "conv"], w[p + "conv.b"])
-    ub = u.view(T, nb, -1)
-    r = torch.sigmoid(torch.einsum("tbi,boi->tbo", ub, w[p + "ra"]) + w[p + "ra.b"]).reshape(T, -1)
-    g = torch.sigmoid(torch.einsum("tbi,boi->tbo", ub, w[p + "ri"]) + w[p + "ri.b"]).reshape(T, -1)
-    log_a = -8.0 * r * torch.nn.functional.softplus(w[p + "lam"])
-    a = torch.exp(log_a)
-    S = torch.zeros(u.shape[1], dtype=F)
-    out = torch.zeros_like(u)
-    for t in range(T):
-        S = a[t] * S + torch.sqrt(1.0 - a[t] ** 2) * g[t] * u[t]
-        out[t] = S
-    return (out * y) @ w[p + "o"].T
+    a, x = rglru_gates(u, w[p + "ra"], w[p + "ra.b"], w[p + "ri"], w[p + "ri.b"], w[p + "lam"])
+    return (linear_scan(a, x) * y) @ w[p + "o"].T
 
 
 def dense_ff(h, w, p, f):
@@ -310,12 +341,16 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int], 
                 x = x + fn(layer_norm(x, nw, nb, eps))
             else:
                 hc = f"l{i}.hc{q}."
-                u = torch.einsum("s,ste->te", w[hc + "in"], xs)
-                y = fn(layer_norm(u, nw, nb, eps))
-                xs = torch.einsum("st,sne->tne", w[hc + "mix"], xs) + w[hc + "out"][:, None, None] * y[None]
+                y = fn(layer_norm(streams_read(xs, w[hc + "in"]), nw, nb, eps))
+                xs = streams_write(xs, y, w[hc + "mix"], w[hc + "out"])
         if layers_out is not None:
             layers_out.append((xs.sum(0) if S is not None else x).clone())
     if S is not None:
         x = xs.sum(0)
     x = layer_norm(x, w["final.norm"], w["final.norm.b"], eps)
     return (x @ w["head"].T) * cfg.get("logit_scale", 1.0)
+
+
+def argmax_first(row) -> int:
+    """The first index of the largest value."""
+    return int((row == row.max()).nonzero()[0])
