@@ -97,73 +97,128 @@ extern "C" int agave_kv_append_rows(int dtype, const void* k, long ldk, const vo
 
 // ------------------------------------------------------------------ q and k rows before they meet
 // 32-bit rows of a step's q, k and v (the projections' results, side by side or apart) become the rows the attention
-// reads and the cache holds: q and k are divided by the root mean square of their whole row (all heads side by side)
-// and multiplied by a weight per element where the mixer has such a norm; the first 2 * half elements of every head
-// are rotated, pair (e, e + half) by the angle pos * freq[e], sine and cosine times `magnitude`; v is only converted.
-// Angles are made in double from double frequencies (a token's sines and cosines once, for all its heads); sums of
-// squares and the rotation are 32-bit.  A workgroup per token.
+// reads and the cache holds: a bias per element is added where the mixer has biases; q and k are divided by the
+// root mean square of their whole row (all heads side by side) and multiplied by a weight per element where the mixer
+// has such a norm; the first 2 * half elements of every head are rotated, pair (e, e + half) by the angle
+// pos * freq[e], sine and cosine times `magnitude`; v is only converted.  k and v go straight into their places in
+// the cache pages (either order) where pages are given, else into rows.
+// The angle is made in double from double frequencies and brought into [-pi, pi] there; its sine and cosine are
+// 32-bit (a token's once, for all its heads); sums of squares and the rotation are 32-bit.  A workgroup per token.
+struct RowsArgs {
+    const float* q; long ldq; const float* k; long ldk; const float* v; long ldv;
+    const float* q_b; const float* k_b; const float* v_b;
+    void* q_out; long ldqo; void* k_out; long ldko; void* v_out; long ldvo;
+    const float* q_w; const float* k_w; float eps_q, eps_k;
+    const double* freq; int half; float magnitude;
+    const int* tok_pos; const int* tok_seq;
+    void* k_pages; void* v_pages; const int* table; int width; const int* base; int head; int n_pages; int packed;
+    int nh, nkv, hd, vd;
+};
+
 template <typename T>
-__global__ __launch_bounds__(256) void row_norm_rope_kernel(const float* __restrict__ q, long ldq, const float* __restrict__ k,
-                                                            long ldk, const float* __restrict__ v, long ldv,
-                                                            T* __restrict__ q_out, long ldqo, T* __restrict__ k_out, long ldko,
-                                                            T* __restrict__ v_out, long ldvo, const float* __restrict__ q_w,
-                                                            const float* __restrict__ k_w, float eps_q, float eps_k,
-                                                            const double* __restrict__ freq, int half, float magnitude,
-                                                            const int* __restrict__ tok_pos, int nh, int nkv, int hd, int vd) {
+__global__ __launch_bounds__(256) void row_norm_rope_kernel(RowsArgs A) {
     __shared__ float cs[2][256];
     __shared__ float red[16];
     const int t = blockIdx.x;
-    const int pos = tok_pos[t];
+    const int pos = A.tok_pos[t];
+    const int half = A.half, hd = A.hd;
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
-        const double ang = (double)pos * freq[i];
-        cs[0][i] = (float)(cos(ang) * (double)magnitude);
-        cs[1][i] = (float)(sin(ang) * (double)magnitude);
+        double ang = (double)pos * A.freq[i];
+        ang -= 6.283185307179586476925 * rint(ang * 0.15915494309189533577);
+        float sn, c;
+        sincosf((float)ang, &sn, &c);
+        cs[0][i] = c * A.magnitude;
+        cs[1][i] = sn * A.magnitude;
     }
+    // where this token's key and value rows live
+    long pg = -1;
+    int prow = 0;
+    if (A.k_pages && A.k) {
+        const int sb = A.tok_seq[t];
+        const int col = page_col(pos / AGAVE_PAGE, A.base[sb], A.head);
+        if (col >= 0 && col < A.width) pg = A.table[(size_t)sb * A.width + col];
+        if (pg >= A.n_pages) pg = -1;
+        prow = pos % AGAVE_PAGE;
+    }
+    const int ksl = (hd + 31) / 32;
+    const size_t kblock = A.packed ? (size_t)AGAVE_PAGE * ksl * 32 : (size_t)AGAVE_PAGE * hd;
     for (int side = 0; side < 2; ++side) {
-        const float* x = side == 0 ? q + (size_t)t * ldq : (k ? k + (size_t)t * ldk : nullptr);
+        const float* x = side == 0 ? A.q + (size_t)t * A.ldq : (A.k ? A.k + (size_t)t * A.ldk : nullptr);
         if (!x) continue;                                   // (the whole workgroup: a run that appends nothing has no k)
-        T* y = side == 0 ? q_out + (size_t)t * ldqo : k_out + (size_t)t * ldko;
-        const float* w = side == 0 ? q_w : k_w;
-        const int heads = side == 0 ? nh : nkv, n = heads * hd;
+        const float* bias = side == 0 ? A.q_b : A.k_b;
+        const float* w = side == 0 ? A.q_w : A.k_w;
+        const int heads = side == 0 ? A.nh : A.nkv, n = heads * hd;
+        const bool to_pages = side == 1 && A.k_pages;
+        T* y = side == 0 ? (T*)A.q_out + (size_t)t * A.ldqo : (to_pages ? nullptr : (T*)A.k_out + (size_t)t * A.ldko);
         float inv = 1.f;
         if (w) {
             float sq = 0.f;
-            for (int i = threadIdx.x; i < n; i += blockDim.x) sq = fmaf(x[i], x[i], sq);
-            inv = 1.0f / sqrtf(block_sum(sq, red) / (float)n + (side == 0 ? eps_q : eps_k));
+            for (int i = threadIdx.x; i < n; i += blockDim.x) {
+                const float v = x[i] + (bias ? bias[i] : 0.f);
+                sq = fmaf(v, v, sq);
+            }
+            inv = 1.0f / sqrtf(block_sum(sq, red) / (float)n + (side == 0 ? A.eps_q : A.eps_k));
         } else {
             __syncthreads();                                // (the table of sines and cosines is complete)
         }
+        auto put = [&](int i, float v) {
+            if (!to_pages) {
+                st(y + i, v);
+            } else if (pg >= 0) {
+                const int g = i / hd, d = i % hd;
+                st((T*)A.k_pages + ((size_t)pg * A.nkv + g) * kblock + (A.packed ? k_operand_at(prow, d, ksl) : (size_t)prow * hd + d), v);
+            }
+        };
         for (int i = threadIdx.x; i < n; i += blockDim.x) {
             const int e = i % hd;
             if (e < half) {
-                const float a = x[i] * inv * (w ? w[i] : 1.f), b = x[i + half] * inv * (w ? w[i + half] : 1.f);
+                const float a = (x[i] + (bias ? bias[i] : 0.f)) * inv * (w ? w[i] : 1.f);
+                const float b = (x[i + half] + (bias ? bias[i + half] : 0.f)) * inv * (w ? w[i + half] : 1.f);
                 const float c = cs[0][e], sn = cs[1][e];
-                st(y + i, a * c - b * sn);
-                st(y + i + half, b * c + a * sn);
+                put(i, a * c - b * sn);
+                put(i + half, b * c + a * sn);
             } else if (e >= 2 * half) {
-                st(y + i, x[i] * inv * (w ? w[i] : 1.f));
+                put(i, (x[i] + (bias ? bias[i] : 0.f)) * inv * (w ? w[i] : 1.f));
             }
         }
     }
-    if (v)
-        for (int i = threadIdx.x; i < nkv * vd; i += blockDim.x) st(v_out + (size_t)t * ldvo + i, v[(size_t)t * ldv + i]);
+    if (A.k && A.v) {
+        const int vd = A.vd;
+        for (int i = threadIdx.x; i < A.nkv * vd; i += blockDim.x) {
+            const float v = A.v[(size_t)t * A.ldv + i] + (A.v_b ? A.v_b[i] : 0.f);
+            if (!A.v_pages) {
+                st((T*)A.v_out + (size_t)t * A.ldvo + i, v);
+            } else if (pg >= 0) {
+                const int g = i / vd, d = i % vd;
+                st((T*)A.v_pages + ((size_t)pg * A.nkv + g) * vd * AGAVE_PAGE + (A.packed ? v_operand_at(d, prow) : (size_t)d * AGAVE_PAGE + prow), v);
+            }
+        }
+    }
 }
 
 extern "C" int agave_row_norm_rope(int dtype, const float* q, long ldq, const float* k, long ldk, const float* v, long ldv,
+                                   const float* q_b, const float* k_b, const float* v_b,
                                    void* q_out, long ldqo, void* k_out, long ldko, void* v_out, long ldvo, const float* q_w,
                                    const float* k_w, float eps_q, float eps_k, const double* freq, int half, float magnitude,
-                                   const int* tok_pos, int N, int nh, int nkv, int hd, int vd, hipStream_t stream) {
+                                   const int* tok_pos, const int* tok_seq, void* k_pages, void* v_pages, const int* table,
+                                   int width, const int* base, int head, int n_pages, int packed,
+                                   int N, int nh, int nkv, int hd, int vd, hipStream_t stream) {
     AGAVE_CHECK(N >= 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0, "row_norm_rope: bad sizes");
     AGAVE_CHECK(q && q_out && tok_pos && ldq >= (long)nh * hd && ldqo >= (long)nh * hd, "row_norm_rope: q rows missing or too short");
-    AGAVE_CHECK(!k || (v && k_out && v_out && ldk >= (long)nkv * hd && ldko >= (long)nkv * hd && ldv >= (long)nkv * vd &&
-                       ldvo >= (long)nkv * vd), "row_norm_rope: k and v rows missing or too short");
+    AGAVE_CHECK(!k || (v && ldk >= (long)nkv * hd && ldv >= (long)nkv * vd), "row_norm_rope: k and v rows missing or too short");
+    AGAVE_CHECK(!k || k_pages || (k_out && v_out && ldko >= (long)nkv * hd && ldvo >= (long)nkv * vd),
+                "row_norm_rope: no place for the k and v rows");
+    AGAVE_CHECK(!k_pages || (v_pages && table && base && tok_seq && width > 0 && n_pages > 0 && head >= 0),
+                "row_norm_rope: cache pages without their table");
+    AGAVE_CHECK(!packed || (dtype == AGAVE_BF16 && hd % 8 == 0 && vd % 16 == 0), "row_norm_rope: pages in operand order hold bfloat16, keys in steps of 8 and values in steps of 16");
     AGAVE_CHECK(half >= 0 && half <= 256 && 2 * half <= hd && (half == 0 || freq), "row_norm_rope: %d rotated pairs in a head of %d (at most 256, with their frequencies)", half, hd);
     if (N == 0) return 0;
-#define RNR_GO(T_) row_norm_rope_kernel<T_><<<N, 256, 0, stream>>>(q, ldq, k, ldk, k ? v : nullptr, ldv, (T_*)q_out, ldqo, (T_*)k_out, ldko, (T_*)v_out, ldvo, q_w, k_w, eps_q, eps_k, freq, half, magnitude, tok_pos, nh, nkv, hd, vd)
-    if (dtype == AGAVE_F32) RNR_GO(float);
-    else if (dtype == AGAVE_BF16) RNR_GO(bf16);
+    RowsArgs A{q, ldq, k, ldk, k ? v : nullptr, ldv, q_b, k_b, v_b, q_out, ldqo, k_out, ldko, v_out, ldvo, q_w, k_w, eps_q, eps_k,
+               freq, half, magnitude, tok_pos, tok_seq, k ? k_pages : nullptr, k ? v_pages : nullptr, table, width, base, head,
+               n_pages, packed, nh, nkv, hd, vd};
+    if (dtype == AGAVE_F32) row_norm_rope_kernel<float><<<N, 256, 0, stream>>>(A);
+    else if (dtype == AGAVE_BF16) row_norm_rope_kernel<bf16><<<N, 256, 0, stream>>>(A);
     else AGAVE_CHECK(false, "row_norm_rope: unknown dtype %d", dtype);
-#undef RNR_GO
     AGAVE_LAUNCH_CHECK("row_norm_rope");
     return 0;
 }

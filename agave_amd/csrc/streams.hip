@@ -94,6 +94,106 @@ __global__ __launch_bounds__(256) void streams_step_kernel(StreamsArgs A) {
     }
 }
 
+// The same for 1 to 8 streams of a width that is a multiple of 4, with aligned rows: four neighbouring columns a thread
+// (16-byte accesses), the number of streams known when the kernel is compiled (every load is written without a
+// condition and all of a thread's loads leave before the first is used), and as many threads a token as the width
+// has groups of four, so that a step of few tokens is one round of loads, two sums and one round of stores.
+template <int S>
+__global__ __launch_bounds__(1024) void streams_step_fast_kernel(StreamsArgs A) {
+    extern __shared__ float u_row[];                 // [E]
+    __shared__ float coef[S * S + 2 * S];
+    __shared__ float red[16];
+    const int E = A.E, E4 = E >> 2;
+    const int t = A.rows ? A.rows[blockIdx.x] : (int)blockIdx.x;
+    float* mixc = coef;
+    float* wrc = coef + S * S;
+    float* rdc = wrc + S;
+    if (threadIdx.x < S * S) mixc[threadIdx.x] = A.y ? A.mix[threadIdx.x] : 0.f;
+    if (threadIdx.x < S) {
+        wrc[threadIdx.x] = A.y ? A.write[threadIdx.x] : 0.f;
+        rdc[threadIdx.x] = A.read ? A.read[threadIdx.x] : 0.f;
+    }
+    __syncthreads();
+    float4* hx = reinterpret_cast<float4*>(A.h + (size_t)t * S * E);
+    float part = 0.f;
+    for (int c = threadIdx.x; c < E4; c += blockDim.x) {
+        float4 x[S];
+#pragma unroll
+        for (int s = 0; s < S; ++s) x[s] = hx[(size_t)s * E4 + c];
+        float4 u = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (A.y) {
+            float4 y = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (A.y_dtype == AGAVE_F32) {
+                for (int sl = 0; sl < A.y_slices; ++sl) {
+                    const float4 v = *reinterpret_cast<const float4*>((const float*)A.y + (size_t)sl * A.y_slice_stride + (size_t)t * A.ldy + 4 * c);
+                    y.x += v.x; y.y += v.y; y.z += v.z; y.w += v.w;
+                }
+            } else {
+                const uint2 v = *reinterpret_cast<const uint2*>((const bf16*)A.y + (size_t)t * A.ldy + 4 * c);
+                y = make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                                __uint_as_float(v.y & 0xffff0000u));
+            }
+#pragma unroll
+            for (int to = 0; to < S; ++to) {
+                const float wv = wrc[to];
+                float4 v = make_float4(wv * y.x, wv * y.y, wv * y.z, wv * y.w);
+#pragma unroll
+                for (int s = 0; s < S; ++s) {
+                    const float m = mixc[s * S + to];
+                    v.x = fmaf(m, x[s].x, v.x); v.y = fmaf(m, x[s].y, v.y); v.z = fmaf(m, x[s].z, v.z); v.w = fmaf(m, x[s].w, v.w);
+                }
+                if (A.store) hx[(size_t)to * E4 + c] = v;
+                const float r = rdc[to];
+                u.x = fmaf(r, v.x, u.x); u.y = fmaf(r, v.y, u.y); u.z = fmaf(r, v.z, u.z); u.w = fmaf(r, v.w, u.w);
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < S; ++s) {
+                const float r = rdc[s];
+                u.x = fmaf(r, x[s].x, u.x); u.y = fmaf(r, x[s].y, u.y); u.z = fmaf(r, x[s].z, u.z); u.w = fmaf(r, x[s].w, u.w);
+            }
+        }
+        reinterpret_cast<float4*>(u_row)[c] = u;
+        part += (u.x + u.y) + (u.z + u.w);
+    }
+    if (!A.out) return;
+    float mean = 0.f;
+    if (A.norm_kind == 1) mean = block_sum(part, red) / (float)E;
+    float sq = 0.f;
+    for (int c = threadIdx.x; c < E4; c += blockDim.x) {             // (a thread reads back what it wrote itself)
+        const float4 v = reinterpret_cast<const float4*>(u_row)[c];
+        const float a = v.x - mean, b = v.y - mean, cc = v.z - mean, d = v.w - mean;
+        sq += (a * a + b * b) + (cc * cc + d * d);
+    }
+    float inv = 1.f;
+    if (A.norm_kind != 0) inv = 1.0f / sqrtf(block_sum(sq, red) / (float)E + A.eps);
+    const size_t orow = (size_t)blockIdx.x * A.ldo;
+    for (int c = threadIdx.x; c < E4; c += blockDim.x) {
+        const float4 v = reinterpret_cast<const float4*>(u_row)[c];
+        float o[4] = {(v.x - mean) * inv, (v.y - mean) * inv, (v.z - mean) * inv, (v.w - mean) * inv};
+        if (A.norm_kind != 0) {
+            const float4 w = reinterpret_cast<const float4*>(A.w)[c];
+            const float4 b = A.b ? reinterpret_cast<const float4*>(A.b)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+            o[0] = fmaf(o[0], w.x, b.x); o[1] = fmaf(o[1], w.y, b.y); o[2] = fmaf(o[2], w.z, b.z); o[3] = fmaf(o[3], w.w, b.w);
+        }
+        if (A.out_dtype == AGAVE_F32) {
+            *reinterpret_cast<float4*>((float*)A.out + orow + 4 * c) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+            uint2 pk;
+            pk.x = f32x2_to_bf16x2(o[0], o[1]);
+            pk.y = f32x2_to_bf16x2(o[2], o[3]);
+            *reinterpret_cast<uint2*>((bf16*)A.out + orow + 4 * c) = pk;
+        }
+    }
+}
+
+template <int S>
+static void launch_streams_fast(const StreamsArgs& A, int blocks, hipStream_t stream) {
+    int threads = ((A.E / 4) + 63) / 64 * 64;
+    threads = threads < 64 ? 64 : threads > 1024 ? 1024 : threads;
+    streams_step_fast_kernel<S><<<blocks, threads, (size_t)A.E * sizeof(float), stream>>>(A);
+}
+
 extern "C" int agave_streams_step(float* h, int N, int S, int E, const void* y, int y_dtype, long ldy, int y_slices,
                                   long y_slice_stride, const float* mix, const float* write, const float* read, int norm_kind,
                                   const float* w, const float* b, float eps, void* out, int out_dtype, long ldo,
@@ -110,7 +210,23 @@ extern "C" int agave_streams_step(float* h, int N, int S, int E, const void* y, 
     if (blocks <= 0 || (!y && !out)) return 0;
     StreamsArgs A{h, S, E, y, y_dtype, ldy, y_slices, y_slice_stride, mix, write, read, norm_kind, w, b, eps,
                   out, out_dtype, ldo, rows, rows ? 0 : 1};
-    streams_step_kernel<<<blocks, 256, (size_t)E * sizeof(float), stream>>>(A);
+    const bool aligned = E % 4 == 0 && ((uintptr_t)h % 16) == 0 &&
+                         (!y || (ldy % 4 == 0 && y_slice_stride % 4 == 0 && ((uintptr_t)y % 16) == 0)) &&
+                         (!out || (ldo % 4 == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)b % 16) == 0));
+    if (aligned && S <= 8) {
+        switch (S) {
+            case 1: launch_streams_fast<1>(A, blocks, stream); break;
+            case 2: launch_streams_fast<2>(A, blocks, stream); break;
+            case 3: launch_streams_fast<3>(A, blocks, stream); break;
+            case 4: launch_streams_fast<4>(A, blocks, stream); break;
+            case 5: launch_streams_fast<5>(A, blocks, stream); break;
+            case 6: launch_streams_fast<6>(A, blocks, stream); break;
+            case 7: launch_streams_fast<7>(A, blocks, stream); break;
+            default: launch_streams_fast<8>(A, blocks, stream); break;
+        }
+    } else {
+        streams_step_kernel<<<blocks, 256, (size_t)E * sizeof(float), stream>>>(A);
+    }
     AGAVE_LAUNCH_CHECK("streams_step");
     return 0;
 }

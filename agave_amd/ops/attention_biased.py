@@ -32,8 +32,8 @@ kernels.register_signatures(LIBRARY, {
     "agave_kv_append_rows": [_I, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P],
     "agave_attn_biased_plain": [_I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F,
                                 _I, _I, _I, _P, _I, _P, _I, _I, _F, _P],
-    "agave_row_norm_rope": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F, _P, _I, _I, _I,
-                            _I, _I, _P],
+    "agave_row_norm_rope": [_I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F, _P, _P,
+                            _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "agave_attn_biased_mfma_ok": [_I, _I, _I, _I, _I],
     "agave_attn_biased_mfma": [_P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I,
                                _F, _I, _I, _I, _P, _I, _P, _I, _P, _I, _F, _P],
@@ -157,13 +157,16 @@ def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], 
 def row_norm_rope(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], q_out: torch.Tensor,
                   k_out: Optional[torch.Tensor], v_out: Optional[torch.Tensor], q_weight: Optional[torch.Tensor],
                   k_weight: Optional[torch.Tensor], eps_q: float, eps_k: float, freq: Optional[torch.Tensor],
-                  magnitude: float, step, n_heads: int, n_kv: int, head_dim: int, v_head_dim: int) -> None:
+                  magnitude: float, step, n_heads: int, n_kv: int, head_dim: int, v_head_dim: int,
+                  biases=(None, None, None), pages=None) -> None:
     """The 32-bit rows of a step's q, k and v (column slices are fine) into the rows the attention reads and the cache
-    holds, in ``q_out``'s element type: q and k divided by the root mean square of their whole row and multiplied by a
-    weight per element (where a weight is given), then each head's first ``2 * len(freq)`` elements rotated, pair
-    (e, e + len(freq)) by the angle ``pos * freq[e]`` (float64 frequencies), sine and cosine times ``magnitude``; v
-    converted.  ``k`` None: only q (a run that appends nothing)."""
-    _dev(q, k, v, q_out, k_out, v_out, q_weight, k_weight, freq)
+    holds, in ``q_out``'s element type: ``biases`` (float32 vectors for q, k, v; any may be None) added; q and k divided
+    by the root mean square of their whole row and multiplied by a weight per element (where a weight is given), then
+    each head's first ``2 * len(freq)`` elements rotated, pair (e, e + len(freq)) by the angle ``pos * freq[e]`` (float64
+    frequencies), sine and cosine times ``magnitude``; v converted.  ``k`` None: only q (a run that appends nothing).
+    ``pages``: ``(k_pages, v_pages, table, base, kept pages, packed)``: the k and v rows go straight into their places in
+    the cache (as :func:`kv_append_rows` would put them) and ``k_out`` / ``v_out`` are not used."""
+    _dev(q, k, v, q_out, k_out, v_out, q_weight, k_weight, freq, *biases)
     n = step.n_tokens
 
     def f32rows(t, what, cols):
@@ -172,17 +175,29 @@ def row_norm_rope(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
         return t.stride(0)
 
     def outrows(t, what, cols):
-        if t.dtype != q_out.dtype or t.dim() != 2 or t.stride(1) != 1 or tuple(t.shape) != (n, cols):
+        if t is None or t.dtype != q_out.dtype or t.dim() != 2 or t.stride(1) != 1 or tuple(t.shape) != (n, cols):
             raise ValueError(f"row_norm_rope: {what} must be rows [{n}, {cols}] of the result's dtype")
         return t.stride(0)
     qd, kd, vd = n_heads * head_dim, n_kv * head_dim, n_kv * v_head_dim
     ldq, ldqo = f32rows(q, "q", qd), outrows(q_out, "q_out", qd)
     ldk = ldv = ldko = ldvo = 0
+    k_pages = v_pages = table = base = None
+    head = width = n_pages = 0
+    packed = False
     if k is not None:
         ldk, ldv = f32rows(k, "k", kd), f32rows(v, "v", vd)
-        ldko, ldvo = outrows(k_out, "k_out", kd), outrows(v_out, "v_out", vd)
+        if pages is not None:
+            k_pages, v_pages, table, base, head, packed = pages
+            _dev(k_pages, v_pages, table, base)
+            n_pages = _check_row_pages(k_pages, v_pages, n_kv, head_dim, v_head_dim, q_out.dtype, packed)
+            width = _check_table(table, base, head, 0)
+            k_out = v_out = None
+        else:
+            ldko, ldvo = outrows(k_out, "k_out", kd), outrows(v_out, "v_out", vd)
     _f32vec(q_weight, "q weight", qd)
     _f32vec(k_weight, "k weight", kd)
+    for b, what, size in zip(biases, ("q bias", "k bias", "v bias"), (qd, kd, vd)):
+        _f32vec(b, what, size)
     half = 0
     if freq is not None:
         if freq.dtype != torch.float64 or not freq.is_contiguous():
@@ -190,6 +205,9 @@ def row_norm_rope(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
         half = freq.numel()
         if 2 * half > head_dim or half > 256:
             raise ValueError(f"row_norm_rope: {2 * half} rotated elements in a head of {head_dim} (at most 512)")
-    library.call(_lib(), "agave_row_norm_rope", dt(q_out), ptr(q), ldq, ptr(k), ldk, ptr(v), ldv, ptr(q_out), ldqo, ptr(k_out),
-                 ldko, ptr(v_out), ldvo, ptr(q_weight), ptr(k_weight), float(eps_q), float(eps_k), ptr(freq), half,
-                 float(magnitude), ptr(step.tok_pos), n, n_heads, n_kv, head_dim, v_head_dim, stream())
+    library.call(_lib(), "agave_row_norm_rope", dt(q_out), ptr(q), ldq, ptr(k), ldk, ptr(v), ldv, ptr(biases[0]), ptr(biases[1]),
+                 ptr(biases[2]), ptr(q_out), ldqo, ptr(k_out), ldko, ptr(v_out), ldvo, ptr(q_weight), ptr(k_weight),
+                 float(eps_q), float(eps_k), ptr(freq), half, float(magnitude), ptr(step.tok_pos),
+                 ptr(step.tok_seq) if k_pages is not None else None,
+                 ptr(k_pages), ptr(v_pages), ptr(table), width, ptr(base), int(head), n_pages, 1 if packed else 0,
+                 n, n_heads, n_kv, head_dim, v_head_dim, stream())

@@ -95,7 +95,6 @@ class BiasedAttention:
             biases.append(None)
             bounds.append(bounds[-1] + self.ctx)
         self._bounds = tuple(bounds)
-        self.proj = Linear(mats, env, "qkvg", biases=biases)    # one product for everything that reads the mixer's input
         # the norm over whole rows and the rotation: q and k pass a kernel of their own on their way
         self.q_weight = self.k_weight = None
         self.q_eps = self.k_eps = 0.0
@@ -119,6 +118,15 @@ class BiasedAttention:
             raise ValueError("biased attention: rotated pairs are (e, e + rotary_dim / 2)")
         self.magnitude = float(getattr(self.position, "magnitude", 1.0))
         self.prepares_rows = self.q_weight is not None or self.k_weight is not None or self.freq is not None
+        # one product for everything that reads the mixer's input; its biases are added by the kernel that prepares the
+        # rows where there is one, else by the product
+        self.row_biases = (None, None, None)
+        if self.prepares_rows:
+            def vec(b):
+                return b.to(torch.float32).contiguous().to(env.device) if b is not None else None
+            self.row_biases = (vec(biases[0]), vec(biases[1]) if self.own_kv else None, vec(biases[2]) if self.own_kv else None)
+            biases = None
+        self.proj = Linear(mats, env, "qkvg", biases=biases)
         if s.chunk is not None and s.keep_first:
             raise ValueError("biased attention: chunks go without kept first positions")
         self.o = Linear([weights.get(s.o_proj)], env, "attn_o")
@@ -180,13 +188,11 @@ class BiasedAttention:
             proj = self.proj.forward(x, out_dtype=torch.float32, tag="qkvg32")
             cols = ws.columns(proj, self._bounds)
             q = ws.get("attn_q_rows", n, self.qd, x.dtype)
-            k = v = None
-            if self.own_kv:
-                kv = ws.get("attn_kv_rows", n, self.kd + self.vd, x.dtype)
-                k, v = ws.columns(kv, (0, self.kd, self.kd + self.vd))
-            ops.row_norm_rope(cols[0], cols[1] if self.own_kv else None, cols[2] if self.own_kv else None, q, k, v,
+            k = v = None                                        # (k and v go straight into the cache pages)
+            ops.row_norm_rope(cols[0], cols[1] if self.own_kv else None, cols[2] if self.own_kv else None, q, None, None,
                               self.q_weight, self.k_weight, self.q_eps, self.k_eps, self.freq, self.magnitude, step,
-                              s.n_heads, s.n_kv_heads, s.head_dim, s.v_head_dim)
+                              s.n_heads, s.n_kv_heads, s.head_dim, s.v_head_dim, biases=self.row_biases,
+                              pages=(k_pages, v_pages, table, base, head, packed) if self.own_kv else None)
             gate = None
             if s.gate_proj:
                 g32 = cols[3 if self.own_kv else 1]
@@ -198,7 +204,7 @@ class BiasedAttention:
             q = cols[0]
             k, v = (cols[1], cols[2]) if self.own_kv else (None, None)
             gate = cols[3 if self.own_kv else 1] if s.gate_proj else None
-        if self.own_kv:
+        if self.own_kv and k is not None:
             ops.kv_append_rows(k, v, k_pages, v_pages, table, base, head, step, s.n_kv_heads, s.head_dim,
                                s.v_head_dim, packed)
         ctx = ws.get("attn_ctx", n, self.ctx, x.dtype)

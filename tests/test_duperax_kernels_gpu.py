@@ -126,6 +126,32 @@ def test_row_norm_and_rotation(dtype, H, G, d, vd, dims, scaling, normed):
     tol = 2e-6 if dtype == torch.float32 else 6e-3
     assert rel(q_out.view(n, H, d), want_q) < tol and rel(kv[:, :G * d].reshape(n, G, d), want_k) < tol
     assert rel(kv[:, G * d:], w64[:, H * d + G * d:H * d + G * d + G * vd]) < tol
+    # biases added on the way, and k and v straight into cache pages: the same rows as the kernel that appends rows puts there
+    from agave_amd.cache import GroupKey, KVCache
+    from agave_amd.engine.step import StepPlanner
+    key = GroupKey(None, G, d, v_head_dim=vd, layout="rows_vt")
+    qb, kb, vb = torch.randn(H * d, generator=g), torch.randn(G * d, generator=g), torch.randn(G * vd, generator=g)
+    stores = []
+    for fused in (True, False):
+        cache = KVCache({0: key}, {}, 2, {key: 4}, dtype, torch.device(DEV), 256)
+        planner = StepPlanner(cache, 1000, torch.device(DEV))
+        step = planner.plan([cache.alloc_slot()], [[0] * n], "all")
+        kp, vp, packed = cache.pages_of(0)
+        table, base = step.tables[0]
+        qo = torch.empty_like(q_out)
+        if fused:
+            A.row_norm_rope(q, k, v, qo, None, None, qw.to(DEV) if normed else None, kw.to(DEV) if normed else None, eps, eps,
+                            freq, magnitude, step, H, G, d, vd, biases=(qb.to(DEV), kb.to(DEV), vb.to(DEV)),
+                            pages=(kp, vp, table, base, 0, packed))
+        else:
+            rows = torch.empty(n, G * d + G * vd, dtype=dtype, device=DEV)
+            A.row_norm_rope(q + qb.to(DEV), k + kb.to(DEV), v + vb.to(DEV), qo, rows[:, :G * d], rows[:, G * d:],
+                            qw.to(DEV) if normed else None, kw.to(DEV) if normed else None, eps, eps, freq, magnitude, step, H, G, d, vd)
+            A.kv_append_rows(rows[:, :G * d], rows[:, G * d:], kp, vp, table, base, 0, step, G, d, vd, packed)
+        stores.append((qo.float().cpu(), kp.float().cpu().clone(), vp.float().cpu().clone()))
+    for got, ref in zip(*stores):
+        assert float((got - ref).abs().max()) <= (1e-6 if dtype == torch.float32 else 2e-2) * max(1.0, float(ref.abs().max()))
+    assert float(stores[0][1].abs().max()) > 0
     # a run that appends nothing norms and rotates its queries alone
     q2 = torch.empty_like(q_out)
     A.row_norm_rope(q, None, None, q2, None, None, qw.to(DEV) if normed else None, None, eps, eps, freq, magnitude,
@@ -230,10 +256,18 @@ def test_attention_with_chunks_and_capped_scores(shape, dtype):
 def test_recurrence_gates(W, blocks, wdtype):
     from agave_amd.ops import rglru as R
     g = torch.Generator().manual_seed(W)
-    n, bw = 75, W // blocks
-    wide = torch.randn(n, W + 5, generator=g) * 1.5
+    bw = W // blocks
     w_r, w_i = (torch.randn(blocks, bw, bw, generator=g) * bw ** -0.5).to(wdtype), (torch.randn(blocks, bw, bw, generator=g) * bw ** -0.5).to(wdtype)
     b_r, b_i, lam = torch.randn(blocks, bw, generator=g), torch.randn(blocks, bw, generator=g), torch.randn(W, generator=g) * 2 - 2
+    for n in (75, 1, 9, 16, 17, 64, 65):               # steps of up to 64 tokens run a kernel of their own
+        wide = torch.randn(n, W + 5, generator=g) * 1.5
+        want_a, want_x = P.rglru_gates(wide[:, 2:2 + W].to(F64).contiguous(), w_r.to(F64), b_r.to(F64), w_i.to(F64), b_i.to(F64), lam.to(F64), c=6.0)
+        decay = (6.0 * torch.nn.functional.softplus(lam.to(F64))).float().to(DEV)
+        a, x = torch.empty(n, W, device=DEV), torch.empty(n, W, device=DEV)
+        R.gates(wide.to(DEV)[:, 2:2 + W], w_r.to(DEV), w_i.to(DEV), b_r.reshape(-1).to(DEV), b_i.reshape(-1).to(DEV), decay, a, x)
+        # (bfloat16 matrices with blocks the matrix cores take: the inputs enter as two bfloat16 numbers, exact to 2^-16)
+        split = wdtype == torch.bfloat16 and bw % 32 == 0 and n > 64
+        assert rel(a, want_a) < (2e-5 if split else 3e-6) and rel(x, want_x) < (5e-5 if split else 1e-5), n
     want_a, want_x = P.rglru_gates(wide[:, 2:2 + W].to(F64).contiguous(), w_r.to(F64), b_r.to(F64), w_i.to(F64), b_i.to(F64), lam.to(F64), c=6.0)
     decay = (6.0 * torch.nn.functional.softplus(lam.to(F64))).float().to(DEV)
     a, x = torch.empty(n, W, device=DEV), torch.empty(n, W, device=DEV)
