@@ -102,7 +102,7 @@ extern "C" int agave_kv_append_rows(int dtype, const void* k, long ldk, const vo
 // has such a norm; the first 2 * half elements of every head are rotated, pair (e, e + half) by the angle
 // pos * freq[e], sine and cosine times `magnitude`; v is only converted.  k and v go straight into their places in
 // the cache pages (either order) where pages are given, else into rows.
-// The angle is made in double from double frequencies and brought into [-pi, pi] there; its sine and cosine are
+// The angle is made in double from double frequencies and reduced to [-pi/4, pi/4] there; its sine and cosine are
 // 32-bit (a token's once, for all its heads); sums of squares and the rotation are 32-bit.  A workgroup per token.
 struct RowsArgs {
     const float* q; long ldq; const float* k; long ldk; const float* v; long ldv;
@@ -118,22 +118,29 @@ struct RowsArgs {
 template <typename T>
 __global__ __launch_bounds__(256) void row_norm_rope_kernel(RowsArgs A) {
     __shared__ float cs[2][256];
-    __shared__ float red[16];
+    __shared__ float red[2][4];
     const int t = blockIdx.x;
     const int pos = A.tok_pos[t];
     const int half = A.half, hd = A.hd;
+    const bool has_k = A.k != nullptr;
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
-        double ang = (double)pos * A.freq[i];
-        ang -= 6.283185307179586476925 * rint(ang * 0.15915494309189533577);
-        float sn, c;
-        sincosf((float)ang, &sn, &c);
-        cs[0][i] = c * A.magnitude;
-        cs[1][i] = sn * A.magnitude;
+        // the angle in double, less the nearest multiple of pi/2 (in double too); what is left lies in [-pi/4, pi/4],
+        // where sine and cosine are short 32-bit polynomials (errors of a few 1e-8); the quadrant swaps and negates
+        const double ang = (double)pos * A.freq[i];
+        const double q = rint(ang * 0.63661977236758134308);
+        const float r = (float)(ang - q * 1.57079632679489661923), r2 = r * r;
+        const float sp = fmaf(r * r2, fmaf(r2, fmaf(r2, -1.9515295891e-4f, 8.3321608736e-3f), -1.6666654611e-1f), r);
+        const float cp = fmaf(r2 * r2, fmaf(r2, fmaf(r2, 2.443315711809948e-5f, -1.388731625493765e-3f), 4.166664568298827e-2f),
+                              fmaf(r2, -0.5f, 1.0f));
+        const int quad = (int)((long long)q & 3);
+        const float sn = (quad & 1) ? cp : sp, c = (quad & 1) ? sp : cp;
+        cs[0][i] = ((quad == 1 || quad == 2) ? -c : c) * A.magnitude;
+        cs[1][i] = ((quad & 2) ? -sn : sn) * A.magnitude;
     }
     // where this token's key and value rows live
     long pg = -1;
     int prow = 0;
-    if (A.k_pages && A.k) {
+    if (A.k_pages && has_k) {
         const int sb = A.tok_seq[t];
         const int col = page_col(pos / AGAVE_PAGE, A.base[sb], A.head);
         if (col >= 0 && col < A.width) pg = A.table[(size_t)sb * A.width + col];
@@ -142,25 +149,39 @@ __global__ __launch_bounds__(256) void row_norm_rope_kernel(RowsArgs A) {
     }
     const int ksl = (hd + 31) / 32;
     const size_t kblock = A.packed ? (size_t)AGAVE_PAGE * ksl * 32 : (size_t)AGAVE_PAGE * hd;
+    const float* xq = A.q + (size_t)t * A.ldq;
+    const float* xk = has_k ? A.k + (size_t)t * A.ldk : nullptr;
+    const int nq = A.nh * hd, nk = A.nkv * hd;
+    // both rows' sums of squares in one pass and one meeting of the workgroup (which also completes the table)
+    float sq = 0.f, sk = 0.f;
+    if (A.q_w)
+        for (int i = threadIdx.x; i < nq; i += blockDim.x) {
+            const float v = xq[i] + (A.q_b ? A.q_b[i] : 0.f);
+            sq = fmaf(v, v, sq);
+        }
+    if (A.k_w && has_k)
+        for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+            const float v = xk[i] + (A.k_b ? A.k_b[i] : 0.f);
+            sk = fmaf(v, v, sk);
+        }
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    if ((threadIdx.x & 63) == 0) {
+        red[0][threadIdx.x >> 6] = sq;
+        red[1][threadIdx.x >> 6] = sk;
+    }
+    __syncthreads();
+    const float inv_q = A.q_w ? 1.0f / sqrtf(((red[0][0] + red[0][1]) + (red[0][2] + red[0][3])) / (float)nq + A.eps_q) : 1.f;
+    const float inv_k = (A.k_w && has_k) ? 1.0f / sqrtf(((red[1][0] + red[1][1]) + (red[1][2] + red[1][3])) / (float)nk + A.eps_k) : 1.f;
     for (int side = 0; side < 2; ++side) {
-        const float* x = side == 0 ? A.q + (size_t)t * A.ldq : (A.k ? A.k + (size_t)t * A.ldk : nullptr);
+        const float* x = side == 0 ? xq : xk;
         if (!x) continue;                                   // (the whole workgroup: a run that appends nothing has no k)
         const float* bias = side == 0 ? A.q_b : A.k_b;
         const float* w = side == 0 ? A.q_w : A.k_w;
-        const int heads = side == 0 ? A.nh : A.nkv, n = heads * hd;
+        const int heads = side == 0 ? A.nh : A.nkv;
+        const float inv = side == 0 ? inv_q : inv_k;
         const bool to_pages = side == 1 && A.k_pages;
         T* y = side == 0 ? (T*)A.q_out + (size_t)t * A.ldqo : (to_pages ? nullptr : (T*)A.k_out + (size_t)t * A.ldko);
-        float inv = 1.f;
-        if (w) {
-            float sq = 0.f;
-            for (int i = threadIdx.x; i < n; i += blockDim.x) {
-                const float v = x[i] + (bias ? bias[i] : 0.f);
-                sq = fmaf(v, v, sq);
-            }
-            inv = 1.0f / sqrtf(block_sum(sq, red) / (float)n + (side == 0 ? A.eps_q : A.eps_k));
-        } else {
-            __syncthreads();                                // (the table of sines and cosines is complete)
-        }
         auto put = [&](int i, float v) {
             if (!to_pages) {
                 st(y + i, v);
@@ -169,20 +190,44 @@ __global__ __launch_bounds__(256) void row_norm_rope_kernel(RowsArgs A) {
                 st((T*)A.k_pages + ((size_t)pg * A.nkv + g) * kblock + (A.packed ? k_operand_at(prow, d, ksl) : (size_t)prow * hd + d), v);
             }
         };
-        for (int i = threadIdx.x; i < n; i += blockDim.x) {
-            const int e = i % hd;
-            if (e < half) {
-                const float a = (x[i] + (bias ? bias[i] : 0.f)) * inv * (w ? w[i] : 1.f);
-                const float b = (x[i + half] + (bias ? bias[i + half] : 0.f)) * inv * (w ? w[i + half] : 1.f);
+        // (whether there are biases and weights is known outside the loops, so that no load stands under a condition
+        // and a thread's loads of a pair leave together)
+        auto rows = [&](auto has_b, auto has_w) {
+            constexpr bool HB = decltype(has_b)::value != 0, HW = decltype(has_w)::value != 0;
+            for (int idx = threadIdx.x; idx < heads * half; idx += blockDim.x) {           // the rotated pairs
+                const int e = idx % half, i = (idx / half) * hd + e;
+                float a = x[i], b = x[i + half];
+                if (HB) {
+                    a += bias[i];
+                    b += bias[i + half];
+                }
+                a *= inv;
+                b *= inv;
+                if (HW) {
+                    a *= w[i];
+                    b *= w[i + half];
+                }
                 const float c = cs[0][e], sn = cs[1][e];
                 put(i, a * c - b * sn);
                 put(i + half, b * c + a * sn);
-            } else if (e >= 2 * half) {
-                put(i, (x[i] + (bias ? bias[i] : 0.f)) * inv * (w ? w[i] : 1.f));
             }
+            const int rest = hd - 2 * half;
+            for (int idx = threadIdx.x; idx < heads * rest; idx += blockDim.x) {           // what is not rotated
+                const int i = (idx / rest) * hd + 2 * half + idx % rest;
+                float a = x[i];
+                if (HB) a += bias[i];
+                a *= inv;
+                if (HW) a *= w[i];
+                put(i, a);
+            }
+        };
+        if (bias) {
+            if (w) rows(IntC<1>{}, IntC<1>{}); else rows(IntC<1>{}, IntC<0>{});
+        } else {
+            if (w) rows(IntC<0>{}, IntC<1>{}); else rows(IntC<0>{}, IntC<0>{});
         }
     }
-    if (A.k && A.v) {
+    if (has_k && A.v) {
         const int vd = A.vd;
         for (int i = threadIdx.x; i < A.nkv * vd; i += blockDim.x) {
             const float v = A.v[(size_t)t * A.ldv + i] + (A.v_b ? A.v_b[i] : 0.f);

@@ -246,6 +246,7 @@ extern "C" int agave_rglru_gates(int w_dtype, const float* u, long ldu, const vo
 struct ScanArgs {
     const float* a; const float* x;                  // [N][W]
     const float* y; long ldy;                        // [N][W] (strided): the other branch before its activation
+    const float* y_bias;                             // [W] or null: added before the activation
     void* out; int out_dtype; long ldo;              // [N][W]
     float* state;                                    // [slots][W]
     const int* tok_seq; const int* cu; const int* slots;
@@ -279,12 +280,13 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(ScanArgs A) {
     const int ch = blockIdx.x * blockDim.x + threadIdx.x;
     if (ch >= A.W) return;
     float P = 1.f, S = (MODE == 1 && k > 0) ? A.carry[(size_t)k * A.W + ch] : 0.f;
+    const float yb = (MODE == 1 && A.y_bias) ? A.y_bias[ch] : 0.f;
 #pragma unroll 4
     for (int t = t0; t < t1; ++t) {
         const int f = flags[t - t0];
         const float a = A.a[(size_t)t * A.W + ch], x = A.x[(size_t)t * A.W + ch];
         float y = 0.f;
-        if (MODE == 1) y = A.y[(size_t)t * A.ldy + ch];
+        if (MODE == 1) y = A.y[(size_t)t * A.ldy + ch] + yb;
         if (f & 1) {
             S = A.state[(size_t)slot_of[t - t0] * A.W + ch];
             P = 0.f;
@@ -323,7 +325,7 @@ __global__ __launch_bounds__(256) void rglru_states_kernel(ScanArgs A) {
     if (ch < A.W) A.state[(size_t)A.slots[blockIdx.y] * A.W + ch] = A.fin[(size_t)blockIdx.y * A.W + ch];
 }
 
-extern "C" int agave_rglru_scan(const float* a, const float* x, const float* y, long ldy, void* out, int out_dtype, long ldo,
+extern "C" int agave_rglru_scan(const float* a, const float* x, const float* y, long ldy, const float* y_bias, void* out, int out_dtype, long ldo,
                                 float* state, const int* tok_seq, const int* cu, const int* slots, float* scratch,
                                 long scratch_floats, int N, int n_seqs, int W, int L, hipStream_t stream) {
     AGAVE_CHECK(a && x && y && out && state && tok_seq && cu && slots, "rglru_scan: null buffer");
@@ -332,7 +334,7 @@ extern "C" int agave_rglru_scan(const float* a, const float* x, const float* y, 
     if (N == 0) return 0;
     const int chunks = (N + L - 1) / L;
     AGAVE_CHECK(chunks <= 65535, "rglru_scan: %d chunks of rows", chunks);
-    ScanArgs A{a, x, y, ldy, out, out_dtype, ldo, state, tok_seq, cu, slots, nullptr, nullptr, nullptr, nullptr, N, W, L};
+    ScanArgs A{a, x, y, ldy, y_bias, out, out_dtype, ldo, state, tok_seq, cu, slots, nullptr, nullptr, nullptr, nullptr, N, W, L};
     const dim3 grid((W + 255) / 256, chunks);
     if (chunks > 1) {
         const long need = (3L * chunks + n_seqs) * W;

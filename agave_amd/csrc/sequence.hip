@@ -39,19 +39,20 @@ __global__ void short_conv_kernel(const float* __restrict__ u, long ldu, const f
                                   const float* __restrict__ bias, float* __restrict__ y, long ldy, float* __restrict__ state,
                                   const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                   const int* __restrict__ pos0, const int* __restrict__ slots, int C, int taps,
-                                  int fused_update) {
+                                  int fused_update, const float* __restrict__ in_bias) {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     const int t = blockIdx.y;
     if (c >= C) return;
     const int s = tok_seq[t], p = tok_pos[t], p0 = pos0[s];
     float* st_c = state + ((size_t)slots[s] * (taps - 1)) * C + c;
+    const float ib = in_bias ? in_bias[c] : 0.f;            // added to every input of the step (the state holds inputs with it)
     float in[CONV_MAX_TAPS];
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS; ++j) {
         in[j] = 0.f;
         if (j < taps) {
             const int r = p - taps + 1 + j;                 // position of this tap's input
-            if (r >= p0) in[j] = u[(size_t)(t - (p - r)) * ldu + c];
+            if (r >= p0) in[j] = u[(size_t)(t - (p - r)) * ldu + c] + ib;
             else in[j] = st_c[(size_t)(r - (p0 - (taps - 1))) * C];
         }
     }
@@ -69,7 +70,7 @@ __global__ void short_conv_kernel(const float* __restrict__ u, long ldu, const f
 
 __global__ void conv_state_kernel(const float* __restrict__ u, long ldu, float* __restrict__ state,
                                   const int* __restrict__ cu, const int* __restrict__ pos0,
-                                  const int* __restrict__ slots, int C, int taps) {
+                                  const int* __restrict__ slots, int C, int taps, const float* __restrict__ in_bias) {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     const int s = blockIdx.y;
     if (c >= C) return;
@@ -81,7 +82,7 @@ __global__ void conv_state_kernel(const float* __restrict__ u, long ldu, float* 
         keep[i] = 0.f;
         if (i < taps - 1) {
             const int back = taps - 1 - i;                  // the input `back` positions before the new end
-            if (back <= n) keep[i] = u[(size_t)(r0 + n - back) * ldu + c];
+            if (back <= n) keep[i] = u[(size_t)(r0 + n - back) * ldu + c] + (in_bias ? in_bias[c] : 0.f);
             else keep[i] = st_c[(size_t)(i + n) * C];
         }
     }
@@ -93,7 +94,7 @@ __global__ void conv_state_kernel(const float* __restrict__ u, long ldu, float* 
 extern "C" int agave_short_conv(const float* u, long ldu, const float* w, const float* bias, float* y, long ldy, float* state,
                                 const int* tok_seq, const int* tok_pos, const int* cu, const int* pos0,
                                 const int* slots, int n_tokens, int n_seqs, int C, int taps, int silu,
-                                int one_token_each, hipStream_t stream) {
+                                int one_token_each, const float* in_bias, hipStream_t stream) {
     AGAVE_CHECK(n_tokens >= 0 && n_seqs >= 0 && C > 0, "short_conv: bad sizes N=%d B=%d C=%d", n_tokens, n_seqs, C);
     AGAVE_CHECK(taps >= 1 && taps <= CONV_MAX_TAPS, "short_conv: %d taps (1 to %d are supported)", taps, CONV_MAX_TAPS);
     AGAVE_CHECK(ldu >= C && ldy >= C, "short_conv: a row stride is below %d", C);
@@ -104,12 +105,12 @@ extern "C" int agave_short_conv(const float* u, long ldu, const float* w, const 
     const int threads = C >= 256 ? 256 : 64;
     const dim3 grid((C + threads - 1) / threads, n_tokens);
     if (silu)
-        short_conv_kernel<true><<<grid, threads, 0, stream>>>(u, ldu, w, bias, y, ldy, state, tok_seq, tok_pos, pos0, slots, C, taps, one_token_each);
+        short_conv_kernel<true><<<grid, threads, 0, stream>>>(u, ldu, w, bias, y, ldy, state, tok_seq, tok_pos, pos0, slots, C, taps, one_token_each, in_bias);
     else
-        short_conv_kernel<false><<<grid, threads, 0, stream>>>(u, ldu, w, bias, y, ldy, state, tok_seq, tok_pos, pos0, slots, C, taps, one_token_each);
+        short_conv_kernel<false><<<grid, threads, 0, stream>>>(u, ldu, w, bias, y, ldy, state, tok_seq, tok_pos, pos0, slots, C, taps, one_token_each, in_bias);
     AGAVE_LAUNCH_CHECK("short_conv");
     if (!one_token_each && taps > 1) {
-        conv_state_kernel<<<dim3((C + threads - 1) / threads, n_seqs), threads, 0, stream>>>(u, ldu, state, cu, pos0, slots, C, taps);
+        conv_state_kernel<<<dim3((C + threads - 1) / threads, n_seqs), threads, 0, stream>>>(u, ldu, state, cu, pos0, slots, C, taps, in_bias);
         AGAVE_LAUNCH_CHECK("conv_state");
     }
     return 0;

@@ -12,7 +12,7 @@ CHUNK = 32                     # rows of a step that one thread walks through in
 
 kernels.register_signatures(LIBRARY, {
     "agave_rglru_gates": [_I, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
-    "agave_rglru_scan": [_P, _P, _P, _L, _P, _I, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P],
+    "agave_rglru_scan": [_P, _P, _P, _L, _P, _P, _I, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P],
 })
 
 
@@ -42,10 +42,13 @@ def gates(u: torch.Tensor, w_r: torch.Tensor, w_i: torch.Tensor, b_r: torch.Tens
                  ptr(a_out), ptr(x_out), n, w, blocks, stream())
 
 
-def scan(a: torch.Tensor, x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, state: torch.Tensor, step, workspace) -> None:
+def scan(a: torch.Tensor, x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, state: torch.Tensor, step, workspace,
+         y_bias=None) -> None:
     """``S_t = a_t S_(t-1) + x_t`` along every sequence of the step, from the sequence's ``state`` [slots, W], which is
-    left at the last row's; ``out_t = S_t gelu_tanh(y_t)``.  ``a``, ``x`` contiguous float32 [N, W]; ``y`` float32 rows."""
-    _dev(a, x, y, out, state)
+    left at the last row's; ``out_t = S_t gelu_tanh(y_t + y_bias)``.  ``a``, ``x`` contiguous float32 [N, W]; ``y`` float32
+    rows; ``y_bias`` float32 [W] or None."""
+    _dev(a, x, y, out, state, y_bias)
+    _f32vec(y_bias, "y bias", a.shape[1])
     n, w = a.shape
     if n != step.n_tokens:
         raise ValueError("rglru.scan: a row per token of the step")
@@ -64,6 +67,6 @@ def scan(a: torch.Tensor, x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, s
     if chunks > 1:
         floats = (3 * chunks + step.n_seqs) * w
         scratch = workspace.get("rglru_scan_scratch", 3 * chunks + step.n_seqs, w, torch.float32)
-    library.call(_lib(), "agave_rglru_scan", ptr(a), ptr(x), ptr(y), ldy, ptr(out), dt(out), out.stride(0), ptr(state),
+    library.call(_lib(), "agave_rglru_scan", ptr(a), ptr(x), ptr(y), ldy, ptr(y_bias), ptr(out), dt(out), out.stride(0), ptr(state),
                  ptr(step.tok_seq), ptr(step.cu_dev), ptr(step.slots_dev), ptr(scratch), floats, n, step.n_seqs, w, CHUNK,
                  stream())

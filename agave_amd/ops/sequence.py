@@ -18,7 +18,7 @@ from .kernels import _P, _I, _L, _F, _dev, _f32vec, _i32, dt, ptr, stream
 LIBRARY = "sequence"
 
 kernels.register_signatures(LIBRARY, {
-    "agave_short_conv": [_P, _L, _P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "agave_short_conv": [_P, _L, _P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P],
     "agave_head_norm_rope_rows": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _I, _I, _P, _I, _I, _P, _P,
                                   _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "agave_talk_attention": [_I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I,
@@ -46,11 +46,14 @@ def _f32rows(t: torch.Tensor, what: str, n: int, cols: int) -> int:
 
 
 def short_conv(u: torch.Tensor, weight: torch.Tensor, y: torch.Tensor, state: torch.Tensor, step, silu: bool,
-               bias: Optional[torch.Tensor] = None) -> None:
+               bias: Optional[torch.Tensor] = None, in_bias: Optional[torch.Tensor] = None) -> None:
     """y[t, c] = act(bias[c] + sum_j weight[c, j] * u[t - taps + 1 + j, c]) along each sequence, zeros before its
-    start; ``state`` [slots, taps - 1, C] holds each sequence's last inputs and is advanced."""
-    _dev(u, weight, y, state, bias)
+    start; ``state`` [slots, taps - 1, C] holds each sequence's last inputs and is advanced.  ``in_bias`` [C] is added
+    to every input u[t, c] on the way in (not to the zeros before a sequence's start): the bias of the product
+    that made the inputs, without a kernel of its own."""
+    _dev(u, weight, y, state, bias, in_bias)
     _f32vec(bias, "conv bias", weight.shape[0])
+    _f32vec(in_bias, "conv input bias", weight.shape[0])
     n = step.n_tokens
     c, taps = weight.shape
     ldu, ldy = _f32rows(u, "conv input", n, c), _f32rows(y, "conv output", n, c)
@@ -64,7 +67,7 @@ def short_conv(u: torch.Tensor, weight: torch.Tensor, y: torch.Tensor, state: to
         raise ValueError("short_conv: a slot lies outside the state")
     library.call(_lib(), "agave_short_conv", ptr(u), ldu, ptr(weight), ptr(bias), ptr(y), ldy, ptr(state), ptr(step.tok_seq),
                  ptr(step.tok_pos), ptr(step.cu_dev), ptr(step.pos0_dev), ptr(step.slots_dev), n, step.n_seqs, c, taps,
-                 1 if silu else 0, 1 if step.is_decode else 0, stream())
+                 1 if silu else 0, 1 if step.is_decode else 0, ptr(in_bias), stream())
 
 
 def head_norm_rope_rows(q: Optional[torch.Tensor], k: Optional[torch.Tensor], v: Optional[torch.Tensor],

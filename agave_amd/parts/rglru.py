@@ -32,8 +32,12 @@ class Rglru:
         if s.blocks < 1 or s.width % s.blocks:
             raise ValueError(f"rglru: {s.width} channels do not form {s.blocks} equal blocks")
         self.spec, self.env = spec, env
-        self.proj = Linear([weights.get(s.y_proj), weights.get(s.x_proj)], env, "rglru_in",
-                           biases=[weights.get(s.y_bias) if s.y_bias else None, weights.get(s.x_bias) if s.x_bias else None])
+        # (the branches' biases are added where their rows are read next: by the convolution and by the scan's read-out)
+        self.proj = Linear([weights.get(s.y_proj), weights.get(s.x_proj)], env, "rglru_in")
+
+        def bias(name):
+            return weights.get(name).to(torch.float32).reshape(-1).contiguous().to(env.device) if name else None
+        self.y_bias, self.x_bias = bias(s.y_bias), bias(s.x_bias)
         self.conv = ShortConv([weights.get(s.conv)], env, silu=False, name="rglru_conv",
                               bias=weights.get(s.conv_bias) if s.conv_bias else None)
         if self.conv.channels != s.width:
@@ -78,12 +82,12 @@ class Rglru:
         proj = self.proj.forward(x, out_dtype=torch.float32, tag="rglru_in")
         y, xb = ws.columns(proj, (0, w, 2 * w))
         u = ws.get("rglru_conved", n, w, torch.float32)
-        self.conv.forward(xb, u, state_tensor(step, memory, "conv"), step)
+        self.conv.forward(xb, u, state_tensor(step, memory, "conv"), step, in_bias=self.x_bias)
         a = ws.get("rglru_decay", n, w, torch.float32)
         gx = ws.get("rglru_input", n, w, torch.float32)
         ops.gates(u, self.w_r, self.w_i, self.b_r, self.b_i, self.decay, a, gx)
         ctx = ws.get("rglru_ctx", n, w, self.env.dtype)
-        ops.scan(a, gx, y, ctx, state_tensor(step, memory, "S"), step, ws)
+        ops.scan(a, gx, y, ctx, state_tensor(step, memory, "S"), step, ws, y_bias=self.y_bias)
         return self.o.forward(ctx, tag="rglru_o", slices_ok=True)
 
 

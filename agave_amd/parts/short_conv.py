@@ -39,6 +39,7 @@ class ShortConv:
     def state_need(self) -> StateNeed:
         return StateNeed((self.taps - 1, self.channels), torch.float32)
 
-    def forward(self, u: torch.Tensor, out: torch.Tensor, state: torch.Tensor, step) -> None:
-        """``u`` and ``out``: float32 [N, channels] (column slices are fine); ``state`` is advanced."""
-        seq_ops.short_conv(u, self.weight, out, state, step, self.silu, self.bias)
+    def forward(self, u: torch.Tensor, out: torch.Tensor, state: torch.Tensor, step, in_bias: Optional[torch.Tensor] = None) -> None:
+        """``u`` and ``out``: float32 [N, channels] (column slices are fine); ``state`` is advanced.  ``in_bias``
+        [channels] float32 is added to the inputs on the way in."""
+        seq_ops.short_conv(u, self.weight, out, state, step, self.silu, self.bias, in_bias)

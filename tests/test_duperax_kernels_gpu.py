@@ -294,7 +294,8 @@ def test_recurrence_scan_whole_pieces_tokens_and_ragged_batches(W, dtype):
     a = [torch.rand(T, W, generator=g) ** 0.2 for T in lens]
     x = [torch.randn(T, W, generator=g) for T in lens]
     y = [torch.randn(T, W + 3, generator=g) for T in lens]
-    want = [P.linear_scan(ai.to(F64), xi.to(F64)) * P.gelu_tanh(yi[:, 1:1 + W].to(F64)) for ai, xi, yi in zip(a, x, y)]
+    yb = torch.randn(W, generator=g)
+    want = [P.linear_scan(ai.to(F64), xi.to(F64)) * P.gelu_tanh(yi[:, 1:1 + W].to(F64) + yb.to(F64)) for ai, xi, yi in zip(a, x, y)]
     ws = Workspace(torch.device(DEV))
     tol = 1e-5 if dtype == torch.float32 else 6e-3
 
@@ -306,7 +307,7 @@ def test_recurrence_scan_whole_pieces_tokens_and_ragged_batches(W, dtype):
             step = feed(cache, planner, [slots[i] for i in live], [ranges[i][r][1] - ranges[i][r][0] for i in live])
             cat = lambda ts: torch.cat([ts[members[i]][ranges[i][r][0]:ranges[i][r][1]] for i in live]).to(DEV).contiguous()
             out = torch.empty(step.n_tokens, W, dtype=dtype, device=DEV)
-            R.scan(cat(a), cat(x), cat(y)[:, 1:1 + W], out, cache.state[0], step, ws)
+            R.scan(cat(a), cat(x), cat(y)[:, 1:1 + W], out, cache.state[0], step, ws, y_bias=yb.to(DEV))
             planner.commit(step)
             at = 0
             for i in live:
@@ -327,6 +328,31 @@ def test_recurrence_scan_whole_pieces_tokens_and_ragged_batches(W, dtype):
         got = run(cache, planner, slots, [0, 1, 2], [cuts(lens[m], firsts[m], 1) for m in range(3)])
         for m in range(3):
             assert rel(got[m], want[m]) < tol, (first, piece, m, "together")
+
+
+@pytest.mark.parametrize("taps", [1, 2, 4, 7])
+def test_convolution_with_a_bias_on_its_inputs(taps):
+    """The bias of the product that made the convolution's inputs is added on the way in: to every input of the
+    sequence, not to the zeros before its start, whole, in pieces (also shorter than the taps) and token by token."""
+    from agave_amd.cache import StateNeed
+    from agave_amd.ops import sequence as S
+    C, T = 37, 29
+    g = torch.Generator().manual_seed(taps)
+    u, w = torch.randn(T, C, generator=g), torch.randn(C, taps, generator=g)
+    b_in, b_out = torch.randn(C, generator=g), torch.randn(C, generator=g)
+    ref = P.causal_conv(u.to(F64) + b_in.to(F64), w.to(F64), b_out.to(F64))
+    for first, piece in ((T, 1), (11, 1), (5, 2), (1, 3), (2, 9)):
+        cache, planner = planner_for(state={0: StateNeed((taps - 1, C))})
+        cache.alloc_slot()
+        slot = cache.alloc_slot()
+        got = torch.zeros(T, C)
+        for lo, hi in cuts(T, first, piece):
+            step = feed(cache, planner, [slot], [hi - lo])
+            y = torch.empty(hi - lo, C, device=DEV)
+            S.short_conv(u[lo:hi].to(DEV).contiguous(), w.to(DEV), y, cache.state[0], step, False, b_out.to(DEV), b_in.to(DEV))
+            planner.commit(step)
+            got[lo:hi] = y.cpu()
+        assert rel(got, ref) < 1e-5, (first, piece)
 
 
 # ---------------------------------------------------------------- the router
