@@ -79,8 +79,8 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(const float* __restric
 }
 
 // The same for steps of few tokens (decode steps): a wave per channel, the lanes along the block's inputs, sixteen
-// tokens at a time; the gate matrices' rows stream once, nothing waits in LDS, no load stands under a condition.
-template <typename T>
+// (or eight) tokens at a time; the gate matrices' rows stream once, nothing waits in LDS, no load stands under a condition.
+template <typename T, int NT>
 __global__ __launch_bounds__(256) void rglru_gates_few_kernel(const float* __restrict__ u, long ldu, const T* __restrict__ wr,
                                                               const T* __restrict__ wi, const float* __restrict__ br,
                                                               const float* __restrict__ bi, const float* __restrict__ decay,
@@ -92,16 +92,16 @@ __global__ __launch_bounds__(256) void rglru_gates_few_kernel(const float* __res
     const T* wrr = wr + ((size_t)b * bw + o) * bw;
     const T* wir = wi + ((size_t)b * bw + o) * bw;
     const float rb = br[ch], ib = bi[ch], dc = decay[ch];
-    for (int t0 = 0; t0 < N; t0 += 16) {
-        float ar[16], ai[16];
+    for (int t0 = 0; t0 < N; t0 += NT) {
+        float ar[NT], ai[NT];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) ar[i] = ai[i] = 0.f;
+        for (int i = 0; i < NT; ++i) ar[i] = ai[i] = 0.f;
         for (int k0 = 0; k0 < bw; k0 += 64) {
             const int k = k0 + lane < bw ? k0 + lane : bw - 1;
             const float live = k0 + lane < bw ? 1.f : 0.f;
             const float a = ld(wrr + k) * live, c = ld(wir + k) * live;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
+            for (int i = 0; i < NT; ++i) {
                 const float x = u[(size_t)(t0 + i < N ? t0 + i : N - 1) * ldu + (size_t)b * bw + k];
                 ar[i] = fmaf(a, x, ar[i]);
                 ai[i] = fmaf(c, x, ai[i]);
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(256) void rglru_gates_few_kernel(const float* __res
         }
         float zr = 0.f, zi = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i = 0; i < NT; ++i) {
             const float r = wave_sum(ar[i]), g = wave_sum(ai[i]);
             if (lane == i) {
                 zr = r;
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void rglru_gates_few_kernel(const float* __res
             }
         }
         const int t = t0 + lane;
-        if (lane < 16 && t < N) {
+        if (lane < NT && t < N) {
             const float r = 1.0f / (1.0f + expf(-(zr + rb)));
             const float g = 1.0f / (1.0f + expf(-(zi + ib)));
             const float log_a = -dc * r;
@@ -215,10 +215,13 @@ extern "C" int agave_rglru_gates(int w_dtype, const float* u, long ldu, const vo
     AGAVE_CHECK(grid.y <= 65535 && grid.z <= 65535, "rglru_gates: too many blocks");
     if (N <= 64) {
         const int blocks = (W + 3) / 4;
-        if (w_dtype == AGAVE_F32)
-            rglru_gates_few_kernel<float><<<blocks, 256, 0, stream>>>(u, ldu, (const float*)wr, (const float*)wi, br, bi, decay, a_out, x_out, N, W, bw);
-        else if (w_dtype == AGAVE_BF16)
-            rglru_gates_few_kernel<bf16><<<blocks, 256, 0, stream>>>(u, ldu, (const bf16*)wr, (const bf16*)wi, br, bi, decay, a_out, x_out, N, W, bw);
+#define GATES_FEW(T_, NT_) rglru_gates_few_kernel<T_, NT_><<<blocks, 256, 0, stream>>>(u, ldu, (const T_*)wr, (const T_*)wi, br, bi, decay, a_out, x_out, N, W, bw)
+        if (w_dtype == AGAVE_F32) {
+            if (N <= 8) GATES_FEW(float, 8); else GATES_FEW(float, 16);
+        } else if (w_dtype == AGAVE_BF16) {
+            if (N <= 8) GATES_FEW(bf16, 8); else GATES_FEW(bf16, 16);
+        }
+#undef GATES_FEW
         else
             AGAVE_CHECK(false, "rglru_gates: unknown dtype %d", w_dtype);
         AGAVE_LAUNCH_CHECK("rglru_gates");
@@ -279,7 +282,7 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(ScanArgs A) {
     __syncthreads();
     const int ch = blockIdx.x * blockDim.x + threadIdx.x;
     if (ch >= A.W) return;
-    float P = 1.f, S = (MODE == 1 && k > 0) ? A.carry[(size_t)k * A.W + ch] : 0.f;
+    float P = 1.f, S = (MODE == 1 && k > 0 && A.carry) ? A.carry[(size_t)k * A.W + ch] : 0.f;
     const float yb = (MODE == 1 && A.y_bias) ? A.y_bias[ch] : 0.f;
 #pragma unroll 4
     for (int t = t0; t < t1; ++t) {
@@ -310,11 +313,25 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(ScanArgs A) {
 }
 
 // carry[k] = what enters chunk k: carry[k + 1] = P[k] carry[k] + Q[k] (chunk 0 always starts at a sequence's first row)
-__global__ __launch_bounds__(256) void rglru_carry_kernel(ScanArgs A, int chunks) {
+__global__ __launch_bounds__(64) void rglru_carry_kernel(ScanArgs A, int chunks) {
     const int ch = blockIdx.x * blockDim.x + threadIdx.x;
     if (ch >= A.W) return;
     float S = 0.f;
-    for (int k = 0; k + 1 < chunks; ++k) {
+    int k = 0;
+    for (; k + 8 < chunks; k += 8) {                   // eight chunks' (P, Q) asked for at once, then the chain
+        float p[8], q[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            p[i] = A.P[(size_t)(k + i) * A.W + ch];
+            q[i] = A.Q[(size_t)(k + i) * A.W + ch];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            S = fmaf(p[i], S, q[i]);
+            A.carry[(size_t)(k + i + 1) * A.W + ch] = S;
+        }
+    }
+    for (; k + 1 < chunks; ++k) {
         S = fmaf(A.P[(size_t)k * A.W + ch], S, A.Q[(size_t)k * A.W + ch]);
         A.carry[(size_t)(k + 1) * A.W + ch] = S;
     }
@@ -327,11 +344,19 @@ __global__ __launch_bounds__(256) void rglru_states_kernel(ScanArgs A) {
 
 extern "C" int agave_rglru_scan(const float* a, const float* x, const float* y, long ldy, const float* y_bias, void* out, int out_dtype, long ldo,
                                 float* state, const int* tok_seq, const int* cu, const int* slots, float* scratch,
-                                long scratch_floats, int N, int n_seqs, int W, int L, hipStream_t stream) {
+                                long scratch_floats, int N, int n_seqs, int W, int L, int one_row_each, hipStream_t stream) {
     AGAVE_CHECK(a && x && y && out && state && tok_seq && cu && slots, "rglru_scan: null buffer");
     AGAVE_CHECK(N >= 0 && W > 0 && L > 0 && L <= SCAN_MAX_L && ldy >= W && ldo >= W, "rglru_scan: bad sizes N=%d W=%d L=%d", N, W, L);
     AGAVE_CHECK(out_dtype == AGAVE_F32 || out_dtype == AGAVE_BF16, "rglru_scan: unknown dtype %d", out_dtype);
     if (N == 0) return 0;
+    if (one_row_each) {
+        // every row is a sequence's first and last of the step: a chunk a row, each from its slot's state and back to it
+        AGAVE_CHECK(N == n_seqs && N <= 65535, "rglru_scan: a step of one row a sequence has as many rows as sequences");
+        ScanArgs E{a, x, y, ldy, y_bias, out, out_dtype, ldo, state, tok_seq, cu, slots, nullptr, nullptr, nullptr, nullptr, N, W, 1};
+        rglru_scan_kernel<1><<<dim3((W + 255) / 256, N), 256, 0, stream>>>(E);
+        AGAVE_LAUNCH_CHECK("rglru_scan");
+        return 0;
+    }
     const int chunks = (N + L - 1) / L;
     AGAVE_CHECK(chunks <= 65535, "rglru_scan: %d chunks of rows", chunks);
     ScanArgs A{a, x, y, ldy, y_bias, out, out_dtype, ldo, state, tok_seq, cu, slots, nullptr, nullptr, nullptr, nullptr, N, W, L};
@@ -344,7 +369,7 @@ extern "C" int agave_rglru_scan(const float* a, const float* x, const float* y, 
         A.Q = scratch + (size_t)chunks * W;
         A.carry = scratch + 2 * (size_t)chunks * W;
         rglru_scan_kernel<0><<<grid, 256, 0, stream>>>(A);
-        rglru_carry_kernel<<<(W + 255) / 256, 256, 0, stream>>>(A, chunks);
+        rglru_carry_kernel<<<(W + 63) / 64, 64, 0, stream>>>(A, chunks);
     }
     rglru_scan_kernel<1><<<grid, 256, 0, stream>>>(A);
     if (A.fin) rglru_states_kernel<<<dim3((W + 255) / 256, n_seqs), 256, 0, stream>>>(A);

@@ -12,7 +12,7 @@ CHUNK = 32                     # rows of a step that one thread walks through in
 
 kernels.register_signatures(LIBRARY, {
     "agave_rglru_gates": [_I, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
-    "agave_rglru_scan": [_P, _P, _P, _L, _P, _P, _I, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P],
+    "agave_rglru_scan": [_P, _P, _P, _L, _P, _P, _I, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P],
 })
 
 
@@ -62,11 +62,13 @@ def scan(a: torch.Tensor, x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, s
         raise ValueError(f"rglru.scan: state must be contiguous float32 [slots, {w}]")
     if max(step.slots) >= state.shape[0]:
         raise ValueError("rglru.scan: a slot lies outside the state")
+    # a step of one row a sequence (every decode step): the rows do not depend on each other
+    one_each = bool(step.is_decode and n == step.n_seqs)
     chunks = (n + CHUNK - 1) // CHUNK
     scratch, floats = None, 0
-    if chunks > 1:
+    if chunks > 1 and not one_each:
         floats = (3 * chunks + step.n_seqs) * w
         scratch = workspace.get("rglru_scan_scratch", 3 * chunks + step.n_seqs, w, torch.float32)
     library.call(_lib(), "agave_rglru_scan", ptr(a), ptr(x), ptr(y), ldy, ptr(y_bias), ptr(out), dt(out), out.stride(0), ptr(state),
                  ptr(step.tok_seq), ptr(step.cu_dev), ptr(step.slots_dev), ptr(scratch), floats, n, step.n_seqs, w, CHUNK,
-                 stream())
+                 1 if one_each else 0, stream())
