@@ -105,8 +105,9 @@ def tensor_shapes(cfg: dict) -> Dict[str, tuple]:
 
 def random_weights(cfg: dict, seed: int, matrix_std: Optional[float] = None, decided_routing: bool = False) -> Dict[str, torch.Tensor]:
     """Weights that keep activations of order one through many layers, rounded to bfloat16 values (so that a
-    bfloat16 checkpoint holds exactly these numbers).  ``decided_routing``: the corrections of the routers lie two
-    apart, so that no rounding of a score changes which experts are chosen."""
+    bfloat16 checkpoint holds exactly these numbers).  ``decided_routing``: the corrections of the routers are
+    different powers of two (no two pairs of them have the same sum, so groups do not tie either), so that no rounding
+    of a score changes which experts are chosen."""
     g = torch.Generator().manual_seed(seed)
     out = {}
     for name, shape in tensor_shapes(cfg).items():
@@ -126,7 +127,7 @@ def random_weights(cfg: dict, seed: int, matrix_std: Optional[float] = None, dec
         elif last == "correction":
             t = 0.2 * torch.randn(shape, generator=g, dtype=F)
             if decided_routing:
-                t = 2.0 * torch.randperm(shape[0], generator=g).to(F)
+                t = 0.5 * 2.0 ** torch.randperm(shape[0], generator=g).to(F)
         elif last == "conv":
             t = 0.5 * torch.randn(shape, generator=g, dtype=F)
         elif name == "embed":

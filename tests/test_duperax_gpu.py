@@ -283,6 +283,68 @@ def test_an_early_token_stays_in_the_state():
         eng.prefill_chunk = 0
 
 
+def random_config(seed: int) -> dict:
+    """A configuration drawn from a seed: two to five layers of any kind and order, head counts and sizes that the
+    matrix cores take and ones they do not, windows and chunks around page borders, rotations of a part of a head,
+    blocks of the recurrence from 8 to 128 channels, one to eight streams or one ordinary residual, with or without
+    a stretch of layers that runs again."""
+    import random
+    rng = random.Random(seed)
+    layers = []
+    n_layers = rng.randint(2, 5)
+    for _ in range(n_layers):
+        kind = rng.choice(["attention", "attention_2", "rglru"])
+        r = rng.random()
+        if r < 0.2:
+            mlp = None
+        elif r < 0.55:
+            mlp = P.dense(rng.choice([64, 96, 200]), limit=rng.choice([0.5, 1.5, 7.0]))
+        else:
+            groups, per = rng.choice([1, 2, 3, 4]), rng.choice([1, 2, 3, 4])
+            keep = rng.randint(1, groups)
+            mlp = P.moe(groups * per, rng.randint(1, min(keep * per, 6)), groups, keep, rng.choice([32, 48, 96]))
+        if kind == "rglru":
+            blocks = rng.choice([1, 2, 4, 5, 8])
+            layers.append(P.rglru_layer(blocks * rng.choice([8, 20, 32, 64, 128]), blocks, rng.randint(1, 6), mlp=mlp))
+            continue
+        kv = rng.choice([1, 1, 2, 3, 4])
+        heads, dim = kv * rng.choice([1, 2, 3, 4, 8]), rng.choice([8, 16, 24, 48, 64, 80, 128, 20, 36])
+        vdim = rng.choice([dim, 16, 32, 48, 24, 40])
+        size = rng.choice([1, 2, 7, 31, 63, 64, 65, 72, 100, 127, 128, 129, 200, 400])
+        scale = rng.choice([dim ** -0.5, 0.125, 1.7 * dim ** -0.5])
+        if kind == "attention":
+            layers.append(P.attention_layer(heads, kv, dim, vdim, size, scale=scale, mlp=mlp))
+        else:
+            dims = max(2, rng.choice([dim, dim // 2, 2, dim - dim // 4]) // 2 * 2)
+            layers.append(P.attention2_layer(heads, kv, dim, vdim, max(size, 2), dims, base=rng.choice([100.0, 1e4, 1e6]),
+                                             factor=rng.choice([1.0, 2.0, 8.0, 32.0]), original=rng.choice([16, 64, 1024, 4096]),
+                                             fast=rng.choice([32.0, 4.0]), slow=rng.choice([1.0, 0.5]),
+                                             softcap=rng.choice([5.0, 25.0, 50.0]), scale=scale, mlp=mlp))
+    loop = None
+    if rng.random() < 0.6:
+        a = rng.randint(0, n_layers - 1)
+        loop = (a, rng.randint(a, n_layers), rng.randint(1, 3))
+    return P.config(layers, vocab=rng.choice([97, 256, 1000]), width=rng.choice([64, 96, 128, 160, 320, 72, 100]),
+                    eps=rng.choice([1e-6, 1e-5]), streams=rng.choice([None, 1, 2, 3, 4, 5, 8]), loop=loop,
+                    logit_scale=rng.choice([0.5, 1.0, 2.0]))
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13, 14, 15, 16])
+def test_configurations_drawn_at_random(seed):
+    from agave_amd.engine import Engine
+    cfg = random_config(seed)
+    toks = U.random_tokens(330, cfg["vocab"], seed)
+    others = [U.random_tokens(n, cfg["vocab"], seed + 100 + n) for n in (1, 150)]
+    for dtype in ("float32", "bfloat16"):
+        w = P.random_weights(cfg, seed, decided_routing=(dtype == "bfloat16"))
+        eng = Engine.from_tensors(cfg, {k: v.bfloat16() for k, v in w.items()}, dtype=dtype, max_slots=3, max_context=512)
+        ref = P.forward(cfg, w, toks)
+        close(U.run_tail(eng, toks, 140), ref, dtype, f"{cfg}: tail")
+        outs = U.run_batched(eng, [toks] + others, (300, 1, 100))
+        for o, r in zip(outs, [ref] + [P.forward(cfg, w, t) for t in others]):
+            close(o, r, dtype, f"{cfg}: in a batch")
+
+
 @pytest.mark.parametrize("dtype", ["float32"])
 def test_greedy_generation_through_the_entry_point(models, dtype):
     from agave_amd.sampling import SamplingParams
