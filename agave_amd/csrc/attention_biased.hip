@@ -116,9 +116,9 @@ struct RowsArgs {
 };
 
 template <typename T>
-__global__ __launch_bounds__(256) void row_norm_rope_kernel(RowsArgs A) {
+__global__ __launch_bounds__(1024) void row_norm_rope_kernel(RowsArgs A) {
     __shared__ float cs[2][256];
-    __shared__ float red[2][4];
+    __shared__ float red[2][16];
     const int t = blockIdx.x;
     const int pos = A.tok_pos[t];
     const int half = A.half, hd = A.hd;
@@ -171,8 +171,13 @@ __global__ __launch_bounds__(256) void row_norm_rope_kernel(RowsArgs A) {
         red[1][threadIdx.x >> 6] = sk;
     }
     __syncthreads();
-    const float inv_q = A.q_w ? 1.0f / sqrtf(((red[0][0] + red[0][1]) + (red[0][2] + red[0][3])) / (float)nq + A.eps_q) : 1.f;
-    const float inv_k = (A.k_w && has_k) ? 1.0f / sqrtf(((red[1][0] + red[1][1]) + (red[1][2] + red[1][3])) / (float)nk + A.eps_k) : 1.f;
+    float tq = 0.f, tk = 0.f;
+    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) {
+        tq += red[0][i];
+        tk += red[1][i];
+    }
+    const float inv_q = A.q_w ? 1.0f / sqrtf(tq / (float)nq + A.eps_q) : 1.f;
+    const float inv_k = (A.k_w && has_k) ? 1.0f / sqrtf(tk / (float)nk + A.eps_k) : 1.f;
     for (int side = 0; side < 2; ++side) {
         const float* x = side == 0 ? xq : xk;
         if (!x) continue;                                   // (the whole workgroup: a run that appends nothing has no k)
@@ -261,8 +266,10 @@ extern "C" int agave_row_norm_rope(int dtype, const float* q, long ldq, const fl
     RowsArgs A{q, ldq, k, ldk, k ? v : nullptr, ldv, q_b, k_b, v_b, q_out, ldqo, k_out, ldko, v_out, ldvo, q_w, k_w, eps_q, eps_k,
                freq, half, magnitude, tok_pos, tok_seq, k ? k_pages : nullptr, k ? v_pages : nullptr, table, width, base, head,
                n_pages, packed, nh, nkv, hd, vd};
-    if (dtype == AGAVE_F32) row_norm_rope_kernel<float><<<N, 256, 0, stream>>>(A);
-    else if (dtype == AGAVE_BF16) row_norm_rope_kernel<bf16><<<N, 256, 0, stream>>>(A);
+    // (few tokens: sixteen waves a token, so that a thread has two or three elements and the waves hide each other's waits)
+    const int threads = N <= 64 ? 1024 : 256;
+    if (dtype == AGAVE_F32) row_norm_rope_kernel<float><<<N, threads, 0, stream>>>(A);
+    else if (dtype == AGAVE_BF16) row_norm_rope_kernel<bf16><<<N, threads, 0, stream>>>(A);
     else AGAVE_CHECK(false, "row_norm_rope: unknown dtype %d", dtype);
     AGAVE_LAUNCH_CHECK("row_norm_rope");
     return 0;
